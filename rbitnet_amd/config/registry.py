@@ -19,6 +19,7 @@ from typing import Any, Dict, Iterable, Optional, Tuple
 from ..errors import ConfigError
 from .bagonex import BagonexConfig
 from .llama import LlamaConfig
+from .pulunex import PulunexConfig
 from .tigutar import TigutarConfig
 from .spec import ModelSpec
 
@@ -97,3 +98,4 @@ def load_config(path_or_dict: Any, tensor_names: Optional[Iterable[str]] = None,
 register_architecture("LlamaForCausalLM", LlamaConfig)
 register_architecture("Bagonex", BagonexConfig)
 register_architecture("Tigutar", TigutarConfig)
+register_architecture("Pulunex", PulunexConfig)

@@ -68,7 +68,8 @@ int rb_gemm_bf16(const void* a, const void* w, int w_layout, void* c, int dtype_
 
 // rb_gemm_bf16 with an activation on the way out (epilogue 0 only): act holds xIELU's two numbers (p, q), and
 // C = xIELU(A W^T) with xIELU(z) = softplus(p) z^2 + z/2 for z > 0, (1/2 + softplus(q)) (exp(z) - 1 - z) + z/2 otherwise,
-// applied to the float32 sums before they are stored.  act null: rb_gemm_bf16.
+// applied to the float32 sums before they are stored.  act null: rb_gemm_bf16.  An act[0] that is no number (NaN) asks for
+// the tanh form of GELU instead, z / 2 (1 + tanh(sqrt(2 / pi) (z + 0.044715 z^3))), which has no numbers of its own.
 int rb_gemm_bf16_act(const void* a, const void* w, int w_layout, void* c, int dtype_out, int epilogue, const float* act,
                      int m, int n, int k, float* workspace, void* stream);
 
@@ -164,7 +165,7 @@ int rb_streams_update_layernorm(float* x, int n_streams, long long stream_stride
                                 int out_dtype, void* stream);      // rb_streams_update (mix null: none), then the norm, in one pass
 int rb_streams_update(float* x, int n_streams, long long stream_stride, const float* mix, const float* out_coef, const float* y,
                       const float* scale, int n_tokens, int width, void* stream);
-// out = z > 0 ? softplus(act[0]) z^2 + z/2 : (1/2 + softplus(act[1])) (exp(z) - 1 - z) + z/2
+// out = z > 0 ? softplus(act[0]) z^2 + z/2 : (1/2 + softplus(act[1])) (exp(z) - 1 - z) + z/2; act[0] NaN: the tanh form of GELU
 int rb_xielu(const float* z, const float* act, void* out, int out_dtype, long long n, void* stream);
 // x <- cap * tanh(x / cap)
 int rb_tanh_cap(float* x, float cap, long long n, void* stream);
@@ -244,8 +245,40 @@ int rb_route_top(const float* z, long long z_stride, int n_experts, int top, int
 int rb_routed_experts(const void* h, int dtype, const float* weight, int top, const int32_t* row_pair, const int32_t* tile_expert,
                       int max_rows, const void* w_gate, const void* w_up, const void* w_down, int w_layout, void* y, float* out,
                       int n_experts, int width, int ff, float limit, float alpha, void* stream);
+// rb_route_top with its choices spelled out.  The router has n_outputs outputs, of which the first n_experts are experts
+// with matrices; a pair whose output lies behind them belongs to no run (rb_experts_combine gives it the token's input).
+// score 0: weight = sigmoid(z) of the chosen, chosen by z.  score 1: weight = softmax(z) over all outputs, chosen by
+// softmax + correction (float32 [n_outputs], null: nothing added).
+int rb_route_choose(const float* z, long long z_stride, int n_outputs, int n_experts, int top, int score, const float* correction,
+                    int32_t* sel, float* weight, int32_t* row_pair, int32_t* tile_expert, int max_rows, int n_tokens, void* stream);
+// rb_routed_experts takes weight null (the input is not scaled) and limit <= 0 (no clamps, the plain gate:
+// out[p] = Wd (silu(Wg x) * (Wu x))).
+// out[t] = sum over k of weight[p] * (sel[p] < n_experts ? pairs[p] : h[t]), p = t * top + k, in the order of k; with
+// shared (float32 [T, width]) also + sigmoid(gate[t * gate_stride]) * shared[t].  h of h_dtype [T, width].
+int rb_experts_combine(const float* pairs, const int32_t* sel, const float* weight, int top, int n_experts, const void* h,
+                       int h_dtype, const float* shared, const float* gate, long long gate_stride, float* out, int n_tokens,
+                       int width, void* stream);
 // out[t] = sum over k of pairs[t * top + k], in the order of k.
 int rb_pairs_sum(const float* pairs, int top, float* out, int n_tokens, int width, void* stream);
+
+// ---- attention whose heads' scores are mixed before the softmax, and what stands around it (talking.hip)
+// x[t, :] = table[ids[t], :] * scale + positions[tok_pos[t], :] (positions of the table's dtype, null: none), float32.
+int rb_embed_scaled_pos(const void* table, int table_dtype, const int32_t* ids, float scale, const void* positions,
+                        const int32_t* tok_pos, float* x, int n_tokens, int width, void* stream);
+// x <- s x
+int rb_scale(float* x, float s, long long n, void* stream);
+// rb_rope_store without a rotation, with a bias (float32, laid out like a row of qkv; null: none) added first and, norm != 0,
+// every query and key head divided by sqrt(mean(head^2) + eps).  k_pages null: the row holds query heads only.
+int rb_bias_norm_store(const float* qkv, long long row_width, const float* bias, int norm, float eps, void* q_out, void* k_pages,
+                       void* v_pages, int cache_dtype, const int32_t* tok_pos, const int32_t* tok_seq, const int32_t* block_table,
+                       int bt_stride, int n_tokens, int n_heads, int n_kv_heads, int dim, int vdim, int pad, void* stream);
+// Causal attention with all heads of a token in one workgroup: score[g, j] = q_g . k_j * scale, mixed[h, j] = sum_g
+// talk[h * Hq + g] score[g, j] (talk float32 [Hq, Hq], null: no mixing), softmax over the keys j <= pos that lie in the
+// token's chunk (chunk > 0: pos / chunk == j / chunk) and among the last `window` (window > 0).  Layouts as
+// rb_attention_generic; Hq <= 64, Hq * head_dim <= 8192.
+int rb_attention_mixed(const void* q, const void* k_pages, const void* v_pages, void* out, int dtype, const int32_t* tok_pos,
+                       const int32_t* tok_seq, const int32_t* block_table, int bt_stride, int n_tokens, int n_heads,
+                       int n_kv_heads, int head_dim, float scale, const float* talk, int chunk, int window, void* stream);
 
 // ---- attention through a latent (latent.hip)
 // Per token: cq = rmsnorm(proj[t, 0:q_rank]) * q_gain -> cq [T, q_rank]; rmsnorm(proj[t, kv_col:+kv_rank]) * kv_gain ->

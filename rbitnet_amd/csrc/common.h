@@ -113,17 +113,28 @@ __device__ __forceinline__ void rotate_pair(float x0, float x1, float c, float s
 // ---------------------------------------------------------------- xIELU
 // act(z) = softplus(p) z^2 + z / 2 for z > 0, (1/2 + softplus(q)) (exp(z) - 1 - z) + z / 2 otherwise; (p, q) are two
 // numbers of the model.  xielu_pair turns them into the two factors once; xielu_value applies them.
+// A p that is no number chooses another activation, which has no numbers of its own: the tanh form of GELU,
+// z / 2 (1 + tanh(sqrt(2 / pi) (z + 0.044715 z^3))), so that every product that applies xIELU where it stores its sums
+// applies that one as well.
 struct XieluPair {
   float ap, an;
 };
 __device__ __forceinline__ XieluPair xielu_pair(const float* __restrict__ act) {
   const float p = act[0], q = act[1];
   XieluPair r;
+  if (p != p) {
+    r.ap = r.an = p;
+    return r;
+  }
   r.ap = p > 20.0f ? p : log1pf(expf(p));
   r.an = 0.5f + (q > 20.0f ? q : log1pf(expf(q)));
   return r;
 }
+__device__ __forceinline__ float gelu_tanh_value(float v) {
+  return 0.5f * v * (1.0f + tanhf(0.7978845608028654f * (v + 0.044715f * v * v * v)));
+}
 __device__ __forceinline__ float xielu_value(float v, float ap, float an) {
+  if (ap != ap) return gelu_tanh_value(v);
   return v > 0.f ? fmaf(ap * v, v, 0.5f * v) : fmaf(an, expm1f(v) - v, 0.5f * v);
 }
 

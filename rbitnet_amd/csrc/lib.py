@@ -105,7 +105,7 @@ class KernelTimes:
         return "\n".join(lines)
 
 
-TIMED_OPS = ("recurrence_prep", "linear_recurrence", "layernorm_residual", "rope_store", "head_gate", "pair_norm_mean",
+TIMED_OPS = ("route_choose", "experts_combine", "embed_scaled_pos", "scale", "bias_norm_store", "attention_mixed", "recurrence_prep", "linear_recurrence", "layernorm_residual", "rope_store", "head_gate", "pair_norm_mean",
              "route_top", "routed_experts", "pairs_sum", "embed_streams", "streams_layernorm", "streams_update", "xielu", "tanh_cap", "short_conv",
              "delta_prep", "delta_rule", "gated_rmsnorm", "latent_norm_store", "heads_linear", "attention_sinks", "embed_gather", "add_rmsnorm", "rope_kv_write", "swiglu", "gemm_generic", "gemm_bf16", "gemm_bf16_terms",
              "gemm_bf16_few", "attention_generic", "attention_prefill_bf16", "attention_decode_bf16",
@@ -176,6 +176,12 @@ class Kernels:
             "rb_route_top": [_P, _L, _I, _I, _P, _P, _P, _P, _I, _I, _P],
             "rb_routed_experts": [_P, _I, _P, _I, _P, _P, _I, _P, _P, _P, _I, _P, _P, _I, _I, _I, _F, _F, _P],
             "rb_pairs_sum": [_P, _I, _P, _I, _I, _P],
+            "rb_route_choose": [_P, _L, _I, _I, _I, _I, _P, _P, _P, _P, _P, _I, _I, _P],
+            "rb_experts_combine": [_P, _P, _P, _I, _I, _P, _I, _P, _P, _L, _P, _I, _I, _P],
+            "rb_embed_scaled_pos": [_P, _I, _P, _F, _P, _P, _P, _I, _I, _P],
+            "rb_scale": [_P, _F, _L, _P],
+            "rb_bias_norm_store": [_P, _L, _P, _I, _F, _P, _P, _P, _I, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _P],
+            "rb_attention_mixed": [_P, _P, _P, _P, _I, _P, _P, _P, _I, _I, _I, _I, _I, _F, _P, _I, _I, _P],
         }
         for name, args in sig.items():
             fn = getattr(L, name)
@@ -776,7 +782,8 @@ class Kernels:
         n_experts, ff, _ = w_gate.shape
         max_rows = row_pair.shape[0]
         _check(h, "h")
-        _check(weight, "weight", torch.float32, (n * top,))
+        if weight is not None:                   # None: the experts' inputs are not scaled
+            _check(weight, "weight", torch.float32, (n * top,))
         _check(row_pair, "row_pair", torch.int32)
         _check(tile_expert, "tile_expert", torch.int32, (2 * (max_rows // 16),))
         _check(w_gate, "w_gate", h.dtype, (n_experts, ff, width))
@@ -787,6 +794,117 @@ class Kernels:
         self._ok(self._lib.rb_routed_experts(_ptr(h), dtype_code(h.dtype), _ptr(weight), top, _ptr(row_pair), _ptr(tile_expert),
                                              max_rows, _ptr(w_gate), _ptr(w_up), _ptr(w_down), int(bool(w_frag)), _ptr(y), _ptr(out),
                                              n_experts, width, ff, float(limit), float(alpha), self._stream()))
+
+    def route_choose(self, z: torch.Tensor, n_outputs: int, n_experts: int, top: int, score: int,
+                     correction: Optional[torch.Tensor], sel: torch.Tensor, weight: torch.Tensor, row_pair: torch.Tensor,
+                     tile_expert: torch.Tensor) -> None:
+        """`route_top` with its choices spelled out: the router's first n_experts outputs are experts with matrices, the
+        rest stand for the token's own input; score 0 sigmoid, 1 softmax over all outputs with `correction` [n_outputs]
+        added for the choice only."""
+        n = z.shape[0]
+        _check(z, "z", torch.float32)
+        if z.shape[1] < n_outputs or n_experts > n_outputs:
+            raise KernelError("route_choose: rows too short for the router's outputs")
+        max_rows = row_pair.shape[0]
+        if max_rows < self.routed_rows(n, top, n_experts) or max_rows % 16:
+            raise KernelError("route_choose: too little room for the sorted pairs")
+        if correction is not None:
+            _check(correction, "correction", torch.float32, (n_outputs,))
+        _check(sel, "sel", torch.int32, (n * top,))
+        _check(weight, "weight", torch.float32, (n * top,))
+        _check(row_pair, "row_pair", torch.int32, (max_rows,))
+        _check(tile_expert, "tile_expert", torch.int32, (2 * (max_rows // 16),))
+        self._ok(self._lib.rb_route_choose(_ptr(z), z.shape[1], n_outputs, n_experts, top, int(score), _ptr(correction), _ptr(sel),
+                                           _ptr(weight), _ptr(row_pair), _ptr(tile_expert), max_rows, n, self._stream()))
+
+    def experts_combine(self, pairs: torch.Tensor, sel: torch.Tensor, weight: torch.Tensor, top: int, n_experts: int,
+                        h: torch.Tensor, shared: Optional[torch.Tensor], gate: Optional[torch.Tensor], gate_col: int,
+                        out: torch.Tensor) -> None:
+        """out[t] = sum_k weight * (the pair's expert output, or h[t] for an output behind the experts), plus
+        sigmoid(gate[t, gate_col]) * shared[t] when there is a shared expert."""
+        n, width = out.shape
+        _check(pairs, "pairs", torch.float32, (n * top, width))
+        _check(sel, "sel", torch.int32, (n * top,))
+        _check(weight, "weight", torch.float32, (n * top,))
+        _check(h, "h", None, (n, width))
+        _check(out, "out", torch.float32)
+        gate_ptr, stride = None, 0
+        if shared is not None:
+            _check(shared, "shared", torch.float32, (n, width))
+            _check(gate, "gate", torch.float32)
+            if gate.shape[0] != n or not 0 <= gate_col < gate.shape[1]:
+                raise KernelError("experts_combine: the gate's column lies outside its rows")
+            gate_ptr, stride = gate.data_ptr() + 4 * gate_col, gate.shape[1]
+        self._ok(self._lib.rb_experts_combine(_ptr(pairs), _ptr(sel), _ptr(weight), top, n_experts, _ptr(h), dtype_code(h.dtype),
+                                              _ptr(shared), gate_ptr, stride, _ptr(out), n, width, self._stream()))
+
+    # ------------------------------------------------------------------ attention with mixed heads
+    def embed_scaled_pos(self, table: torch.Tensor, ids: torch.Tensor, scale: float, positions: Optional[torch.Tensor],
+                         tok_pos: torch.Tensor, out: torch.Tensor) -> None:
+        n, width = out.shape
+        _check(table, "table")
+        _check(ids, "ids", torch.int32, (n,))
+        _check(tok_pos, "tok_pos", torch.int32, (n,))
+        _check(out, "out", torch.float32)
+        if table.shape[1] != width:
+            raise KernelError("embedding width mismatch")
+        if positions is not None:
+            _check(positions, "positions", table.dtype)
+            if positions.shape[1] != width:
+                raise KernelError("position table width mismatch")
+        self._ok(self._lib.rb_embed_scaled_pos(_ptr(table), dtype_code(table.dtype), _ptr(ids), float(scale), _ptr(positions),
+                                               _ptr(tok_pos), _ptr(out), n, width, self._stream()))
+
+    def scale(self, x: torch.Tensor, s: float) -> None:
+        _check(x, "x", torch.float32)
+        self._ok(self._lib.rb_scale(_ptr(x), float(s), x.numel(), self._stream()))
+
+    def bias_norm_store(self, qkv: torch.Tensor, bias: Optional[torch.Tensor], norm: bool, eps: float, q_out: torch.Tensor,
+                        k_pages, v_pages, tok_pos, tok_seq, block_table, n_heads: int, n_kv: int, dim: int, vdim: int,
+                        pad: int) -> None:
+        """qkv [T, W] float32 (+ bias [W]); query and key heads divided by their root mean square when `norm`; queries to
+        q_out [T, Hq, pad], keys and values to the pages [*, Hk, 64, pad] (None: the rows hold queries only)."""
+        n, width = qkv.shape
+        owns = k_pages is not None
+        need = (n_heads + n_kv) * dim + n_kv * vdim if owns else n_heads * dim
+        _check(qkv, "qkv", torch.float32)
+        if width != need:
+            raise KernelError(f"bias_norm_store: rows of {width} numbers, the heads take {need}")
+        if bias is not None:
+            _check(bias, "bias", torch.float32, (width,))
+        _check(q_out, "q_out", None, (n, n_heads, pad))
+        _check(tok_pos, "tok_pos", torch.int32, (n,))
+        _check(tok_seq, "tok_seq", torch.int32, (n,))
+        if owns:
+            _check(block_table, "block_table", torch.int32)
+            _check(k_pages, "k_pages", q_out.dtype)
+            _check(v_pages, "v_pages", q_out.dtype, k_pages.shape)
+            if tuple(k_pages.shape[1:]) != (n_kv, self.page_size, pad):
+                raise KernelError(f"cache pages have shape {tuple(k_pages.shape)}, expected [*, {n_kv}, {self.page_size}, {pad}]")
+        self._ok(self._lib.rb_bias_norm_store(_ptr(qkv), width, _ptr(bias), int(bool(norm)), float(eps), _ptr(q_out), _ptr(k_pages),
+                                              _ptr(v_pages), dtype_code(q_out.dtype), _ptr(tok_pos), _ptr(tok_seq),
+                                              _ptr(block_table) if owns else None, block_table.shape[1] if owns else 0, n,
+                                              n_heads, n_kv if owns else 0, dim, vdim, pad, self._stream()))
+
+    def attention_mixed(self, q, k_pages, v_pages, out, tok_pos, tok_seq, block_table, n_heads, n_kv, head_dim, scale, talk,
+                        chunk, window) -> None:
+        """All heads of a token together: scores mixed over the heads by talk [Hq, Hq] (None: none) before the softmax, keys
+        limited to the token's chunk (chunk positions counted from 0; 0: no chunks) and to the last `window` (0: all)."""
+        n = q.shape[0]
+        _check(q, "q", None, (n, n_heads, head_dim))
+        _check(k_pages, "k_pages", q.dtype)
+        _check(v_pages, "v_pages", q.dtype, k_pages.shape)
+        if tuple(k_pages.shape[1:]) != (n_kv, self.page_size, head_dim):
+            raise KernelError("cache pages do not match the head counts")
+        _check(out, "out", q.dtype, (n, n_heads * head_dim))
+        _check(tok_pos, "tok_pos", torch.int32, (n,))
+        _check(tok_seq, "tok_seq", torch.int32, (n,))
+        _check(block_table, "block_table", torch.int32)
+        if talk is not None:
+            _check(talk, "talk", torch.float32, (n_heads, n_heads))
+        self._ok(self._lib.rb_attention_mixed(_ptr(q), _ptr(k_pages), _ptr(v_pages), _ptr(out), dtype_code(q.dtype), _ptr(tok_pos),
+                                              _ptr(tok_seq), _ptr(block_table), block_table.shape[1], n, n_heads, n_kv, head_dim,
+                                              float(scale), _ptr(talk), int(chunk or 0), int(window or 0), self._stream()))
 
     def pairs_sum(self, pairs: torch.Tensor, top: int, out: torch.Tensor) -> None:
         n, width = out.shape

@@ -25,8 +25,11 @@
 #define RT_MAX_EXPERTS 1024
 
 // ---------------------------------------------------------------- route
-__global__ void route_kernel(const float* __restrict__ z, size_t z_stride, int n_experts, int top, int32_t* __restrict__ sel,
-                             float* __restrict__ weight, int n_tokens) {
+// score 0: sigmoid(z) of the chosen logit.  score 1: the softmax of z over all outputs; the choice then goes by the
+// softmax plus `correction` (null: nothing added), the weight is the softmax itself.
+__global__ void route_kernel(const float* __restrict__ z, size_t z_stride, int n_experts, int top, int score,
+                             const float* __restrict__ correction, int32_t* __restrict__ sel, float* __restrict__ weight,
+                             int n_tokens) {
   const int t = blockIdx.x * (blockDim.x / RB_WAVE) + threadIdx.x / RB_WAVE;
   if (t >= n_tokens) return;
   const int lane = threadIdx.x & (RB_WAVE - 1);
@@ -37,6 +40,27 @@ __global__ void route_kernel(const float* __restrict__ z, size_t z_stride, int n
     const int e = lane + RB_WAVE * j;
     v[j] = e < n_experts ? z[(size_t)t * z_stride + e] : -INFINITY;
     if (v[j] != v[j]) v[j] = -INFINITY;
+  }
+  float own[PER];                    // score 1: the softmax, kept beside what the choice goes by
+  if (score == 1) {
+    float m = -INFINITY;
+#pragma unroll
+    for (int j = 0; j < PER; ++j) m = fmaxf(m, v[j]);
+    m = wave_max(m);
+    float sum = 0.f;
+#pragma unroll
+    for (int j = 0; j < PER; ++j) {
+      own[j] = v[j] == -INFINITY ? 0.f : expf(v[j] - m);
+      sum += own[j];
+    }
+    sum = wave_sum(sum);
+#pragma unroll
+    for (int j = 0; j < PER; ++j) {
+      const int e = lane + RB_WAVE * j;
+      own[j] = own[j] / sum;
+      if (e < n_experts) v[j] = own[j] + (correction ? correction[e] : 0.f);
+      if (v[j] != v[j]) v[j] = -INFINITY;
+    }
   }
   for (int k = 0; k < top; ++k) {
     float best = -INFINITY;
@@ -59,9 +83,18 @@ __global__ void route_kernel(const float* __restrict__ z, size_t z_stride, int n
       }
     }
     if (at == 0x7fffffff) at = k < n_experts ? k : 0;        // every logit was NaN or -inf: any expert, never out of range
+    if (score == 1) {                   // the chosen output's softmax: from the lane that holds it
+      float w = 0.f;
+#pragma unroll
+      for (int j = 0; j < PER; ++j)
+        if (lane + RB_WAVE * j == at) w = own[j];
+      best = wave_sum(w);
+    } else {
+      best = 1.0f / (1.0f + expf(-best));
+    }
     if (lane == 0) {
       sel[(size_t)t * top + k] = at;
-      weight[(size_t)t * top + k] = 1.0f / (1.0f + expf(-best));
+      weight[(size_t)t * top + k] = best;
     }
 #pragma unroll
     for (int j = 0; j < PER; ++j)
@@ -76,7 +109,8 @@ __global__ __launch_bounds__(1024) void route_sort_kernel(const int32_t* __restr
   __shared__ int counts[RT_MAX_EXPERTS], offs[RT_MAX_EXPERTS], cursor[RT_MAX_EXPERTS];
   for (int e = threadIdx.x; e < n_experts; e += blockDim.x) counts[e] = cursor[e] = 0;
   __syncthreads();
-  for (int p = threadIdx.x; p < n_pairs; p += blockDim.x) atomicAdd(&counts[sel[p]], 1);
+  for (int p = threadIdx.x; p < n_pairs; p += blockDim.x)
+    if (sel[p] < n_experts) atomicAdd(&counts[sel[p]], 1);      // an output behind the experts has no matrices and no run
   for (int r = threadIdx.x; r < max_rows; r += blockDim.x) row_pair[r] = -1;
   for (int i = threadIdx.x; i < max_rows / RT_TILE; i += blockDim.x) tile_expert[i] = -1;
   __syncthreads();
@@ -95,27 +129,39 @@ __global__ __launch_bounds__(1024) void route_sort_kernel(const int32_t* __restr
     }
   for (int p = threadIdx.x; p < n_pairs; p += blockDim.x) {
     const int e = sel[p];
-    row_pair[offs[e] + atomicAdd(&cursor[e], 1)] = p;
+    if (e < n_experts) row_pair[offs[e] + atomicAdd(&cursor[e], 1)] = p;
   }
 }
 
-extern "C" int rb_route_top(const float* z, long long z_stride, int n_experts, int top, int32_t* sel, float* weight,
-                            int32_t* row_pair, int32_t* tile_expert, int max_rows, int n_tokens, void* stream) {
-  RB_RECORDED(rb_route_top(z, z_stride, n_experts, top, sel, weight, row_pair, tile_expert, max_rows, n_tokens, stream));
-  RB_REQUIRE(n_tokens >= 0 && n_experts > 0 && n_experts <= RT_MAX_EXPERTS && top > 0 && top <= n_experts && z_stride >= n_experts,
-             "rb_route_top: bad sizes T=%d experts=%d (at most %d) top=%d", n_tokens, n_experts, RT_MAX_EXPERTS, top);
+extern "C" int rb_route_choose(const float* z, long long z_stride, int n_outputs, int n_experts, int top, int score,
+                               const float* correction, int32_t* sel, float* weight, int32_t* row_pair, int32_t* tile_expert,
+                               int max_rows, int n_tokens, void* stream) {
+  RB_RECORDED(rb_route_choose(z, z_stride, n_outputs, n_experts, top, score, correction, sel, weight, row_pair, tile_expert, max_rows,
+                              n_tokens, stream));
+  RB_REQUIRE(n_tokens >= 0 && n_experts >= 0 && n_outputs >= n_experts && n_outputs > 0 && n_outputs <= RT_MAX_EXPERTS && top > 0 &&
+                 top <= n_outputs && z_stride >= n_outputs,
+             "rb_route_choose: bad sizes T=%d outputs=%d (at most %d) experts=%d top=%d", n_tokens, n_outputs, RT_MAX_EXPERTS, n_experts, top);
+  RB_REQUIRE(score == 0 || score == 1, "rb_route_choose: score %d is neither the sigmoid (0) nor the softmax (1)", score);
+  RB_REQUIRE(correction == nullptr || score == 1, "rb_route_choose: a correction goes with the softmax");
   const long long pairs = (long long)n_tokens * top;
   RB_REQUIRE(max_rows % RT_TILE == 0 && max_rows >= (pairs + RT_TILE - 1) / RT_TILE * RT_TILE + (long long)RT_TILE * n_experts,
-             "rb_route_top: room for %d rows, %lld pairs of %d experts may need more", max_rows, pairs, n_experts);
+             "rb_route_choose: room for %d rows, %lld pairs of %d experts may need more", max_rows, pairs, n_experts);
   if (n_tokens == 0) return 0;
   hipStream_t s = (hipStream_t)stream;
-  route_kernel<<<(n_tokens + 3) / 4, 256, 0, s>>>(z, (size_t)z_stride, n_experts, top, sel, weight, n_tokens);
+  route_kernel<<<(n_tokens + 3) / 4, 256, 0, s>>>(z, (size_t)z_stride, n_outputs, top, score, correction, sel, weight, n_tokens);
   route_sort_kernel<<<1, 1024, 0, s>>>(sel, (int)pairs, n_experts, row_pair, tile_expert, tile_expert + max_rows / RT_TILE, max_rows);
   RB_LAUNCH_CHECK();
   return 0;
 }
 
+extern "C" int rb_route_top(const float* z, long long z_stride, int n_experts, int top, int32_t* sel, float* weight,
+                            int32_t* row_pair, int32_t* tile_expert, int max_rows, int n_tokens, void* stream) {
+  return rb_route_choose(z, z_stride, n_experts, n_experts, top, 0, nullptr, sel, weight, row_pair, tile_expert, max_rows, n_tokens, stream);
+}
+
+// limit > 0: g = min(g, limit), u = clamp(u, +-limit), g sigmoid(alpha g) (u + 1).  limit <= 0: the plain gate silu(g) u.
 __device__ __forceinline__ float gated_unit(float g, float u, float limit, float alpha) {
+  if (!(limit > 0.f)) return g / (1.0f + expf(-g)) * u;
   g = fminf(g, limit);
   u = fminf(fmaxf(u, -limit), limit);
   return g / (1.0f + expf(-alpha * g)) * (u + 1.0f);
@@ -135,7 +181,7 @@ __global__ void routed_up_generic_kernel(const T* __restrict__ h, const float* _
     const int p = row_pair[row];
     if (p < 0) continue;
     const T* x = h + (size_t)(p / top) * width;
-    const float wt = weight[p];
+    const float wt = weight ? weight[p] : 1.0f;
     for (int j = blockIdx.y * n_waves + wave; j < ff; j += gridDim.y * n_waves) {
       const T* gr = w_gate + ((size_t)e * ff + j) * width;
       const T* ur = w_up + ((size_t)e * ff + j) * width;
@@ -186,7 +232,7 @@ __global__ void routed_gather_kernel(const bf16_t* __restrict__ h, const float* 
   const int row = blockIdx.x;
   const int p = row_pair[row];
   if (p < 0) return;
-  const float wt = weight[p];
+  const float wt = weight ? weight[p] : 1.0f;
   const bf16_t* x = h + (size_t)(p / top) * width;
   bf16_t* dst = xs + (size_t)(row / RT_TILE) * RT_TILE * width + 8 * (row % RT_TILE);
   for (int k = 8 * threadIdx.x; k < width; k += 8 * blockDim.x) {
@@ -390,6 +436,48 @@ extern "C" int rb_pairs_sum(const float* pairs, int top, float* out, int n_token
   const size_t n = (size_t)n_tokens * width;
   const size_t blocks = (n + 255) / 256;
   pairs_sum_kernel<<<(int)(blocks < 65535 ? blocks : 65535), 256, 0, (hipStream_t)stream>>>(pairs, top, out, width, n);
+  RB_LAUNCH_CHECK();
+  return 0;
+}
+
+// out[t] = sum over k of weight[p] * (sel[p] < n_experts ? pairs[p] : h[t]), p = t * top + k, in the order of k: the score
+// multiplies the expert's OUTPUT, and an output of the router behind the experts stands for the token's own input.
+// With `shared` (float32 [T, width], what an expert that every token uses gave): + sigmoid(gate[t * gate_stride]) * shared[t].
+template <typename T>
+__global__ void experts_combine_kernel(const float* __restrict__ pairs, const int32_t* __restrict__ sel, const float* __restrict__ weight,
+                                       int top, int n_experts, const T* __restrict__ h, const float* __restrict__ shared,
+                                       const float* __restrict__ gate, size_t gate_stride, float* __restrict__ out, int width) {
+  const int t = blockIdx.x;
+  const float sg = shared ? 1.0f / (1.0f + expf(-gate[(size_t)t * gate_stride])) : 0.f;
+  for (int j = threadIdx.x; j < width; j += blockDim.x) {
+    float v = 0.f;
+    for (int k = 0; k < top; ++k) {
+      const size_t p = (size_t)t * top + k;
+      const float term = sel[p] < n_experts ? pairs[p * width + j] : Num<T>::load(h + (size_t)t * width + j);
+      v = fmaf(weight[p], term, v);
+    }
+    if (shared) v = fmaf(sg, shared[(size_t)t * width + j], v);
+    out[(size_t)t * width + j] = v;
+  }
+}
+
+extern "C" int rb_experts_combine(const float* pairs, const int32_t* sel, const float* weight, int top, int n_experts, const void* h,
+                                  int h_dtype, const float* shared, const float* gate, long long gate_stride, float* out, int n_tokens,
+                                  int width, void* stream) {
+  RB_RECORDED(rb_experts_combine(pairs, sel, weight, top, n_experts, h, h_dtype, shared, gate, gate_stride, out, n_tokens, width, stream));
+  RB_REQUIRE(n_tokens >= 0 && width > 0 && top > 0 && n_experts >= 0, "rb_experts_combine: bad sizes");
+  RB_REQUIRE(shared == nullptr || gate != nullptr, "rb_experts_combine: a shared expert comes with its gate");
+  if (n_tokens == 0) return 0;
+  hipStream_t s = (hipStream_t)stream;
+  const int threads = width >= 256 ? 256 : 64;
+  if (h_dtype == RB_F32)
+    experts_combine_kernel<float><<<n_tokens, threads, 0, s>>>(pairs, sel, weight, top, n_experts, (const float*)h, shared, gate,
+                                                               (size_t)gate_stride, out, width);
+  else if (h_dtype == RB_BF16)
+    experts_combine_kernel<bf16_t><<<n_tokens, threads, 0, s>>>(pairs, sel, weight, top, n_experts, (const bf16_t*)h, shared, gate,
+                                                                (size_t)gate_stride, out, width);
+  else
+    RB_REQUIRE(false, "rb_experts_combine: unknown dtype %d", h_dtype);
   RB_LAUNCH_CHECK();
   return 0;
 }

@@ -18,6 +18,16 @@ names of the matrices relative to the layer's prefix), and three that a plain de
               denominator as exp(sink): no key, no value, not scaled;
   head_gate   True: head h's output is multiplied by sigmoid(Wg h)_h (tensor "gate" [heads, E])
               before the output matrix.
+and four more, each of which sends the layer through the kernels that take all heads of a token together:
+  bias        True: q, k and v have biases (tensors named like the matrices with "_bias": names "q_bias", ...), added
+              to the projections before anything else;
+  qk_norm     None, or {"eps": e}: every query and key head is divided by sqrt(mean(head^2) + e) (no weight); the cache
+              holds the keys as they are then;
+  talk        True: the heads' scores are mixed before the softmax, score_h <- sum_g T[h, g] score_g, with T the tensor
+              "talk" [heads, heads] (float32);
+  chunk       None, or c: a query at position i sees the keys j <= i with i // c == j // c only, chunks being counted
+              from the sequence's first position, whatever a step brings.
+These go without a rotation (position "none") and without a sink.
 A position part that rotates only the first numbers of a head says so with its own head_dim
 (the table's width).  Where keys and values differ in size, or only a part of a head is
 rotated, queries, keys and values are laid out with one head size, the larger of the two,
@@ -46,7 +56,8 @@ from .base import BuildEnv, CacheRequest, Part, TensorSpec, build_part, register
 from .linear import linear, linear_or_terms, linear_to_stream, pack_rows
 
 DEFAULT_NAMES = {"q": "q_proj.weight", "k": "k_proj.weight", "v": "v_proj.weight", "o": "o_proj.weight", "sink": "sink",
-                 "gate": "gate"}
+                 "gate": "gate", "q_bias": "q_proj.bias", "k_bias": "k_proj.bias", "v_bias": "v_proj.bias", "talk": "talk"}
+MIXED_MAX_HEADS, MIXED_MAX_NUMBERS = 64, 8192      # what the kernels that take all heads of a token together hold
 _MATRIX_CORE_HEAD_DIMS = (64, 128)
 _DECODE_GROUPS = tuple(range(1, 17))    # query heads per kv head the decode kernels take
 
@@ -88,6 +99,22 @@ class Attention(Part):
             raise ConfigError(f"attention: a rotation pairs the numbers of a head, {self.rot} of them cannot be paired")
         self.pad = max(self.head_dim, self.value_dim)
         self.same_sizes = self.value_dim == self.head_dim and self.rot in (0, self.head_dim) and self.head_dim % 2 == 0
+        self.has_bias, self.has_talk = bool(params.get("bias")), bool(params.get("talk"))
+        qk_norm = params.get("qk_norm")
+        self.qk_eps = None if qk_norm is None else float(qk_norm["eps"])
+        self.chunk = None if params.get("chunk") is None else int(params["chunk"])
+        if self.chunk is not None and self.chunk <= 0:
+            raise ConfigError("attention: chunk must be positive")
+        # all heads of a token in one workgroup: whenever one of the four is asked for
+        self.mixed = self.has_bias or self.has_talk or self.qk_eps is not None or self.chunk is not None
+        if self.mixed:
+            if self.rot or self.has_sink:
+                raise ConfigError("attention: biases, unit heads, mixed heads and chunks go without a rotation and without a sink")
+            if self.n_heads > MIXED_MAX_HEADS or self.n_heads * self.pad > MIXED_MAX_NUMBERS:
+                raise ConfigError(f"attention: {self.n_heads} heads of {self.pad} numbers are more than the kernels that take all "
+                                  f"heads of a token together hold ({MIXED_MAX_HEADS} heads, {MIXED_MAX_NUMBERS} numbers)")
+        self.bias: Optional[torch.Tensor] = None
+        self.talk: Optional[torch.Tensor] = None
         self.w_gate = None
         self.sink: Optional[torch.Tensor] = None
         self.w_qkv: Optional[torch.Tensor] = None
@@ -102,6 +129,13 @@ class Attention(Part):
         if self.cache_from is None:
             specs[self.names["k"]] = TensorSpec((kd, self.hidden))
             specs[self.names["v"]] = TensorSpec((self.n_kv * self.value_dim, self.hidden))
+        if self.has_bias:
+            specs[self.names["q_bias"]] = TensorSpec((qd,), role="gain", init="normal")
+            if self.cache_from is None:
+                specs[self.names["k_bias"]] = TensorSpec((kd,), role="gain", init="normal")
+                specs[self.names["v_bias"]] = TensorSpec((self.n_kv * self.value_dim,), role="gain", init="normal")
+        if self.has_talk:
+            specs[self.names["talk"]] = TensorSpec((self.n_heads, self.n_heads), role="gain", init="eye_normal")
         if self.has_sink:
             specs[self.names["sink"]] = TensorSpec((self.n_heads,), role="gain", init="normal")
         if self.has_gate:
@@ -126,6 +160,10 @@ class Attention(Part):
             wide[:, :, :self.value_dim] = o.view(o.shape[0], self.n_heads, self.value_dim)
             o = wide.view(o.shape[0], self.n_heads * self.pad)
         self.w_o = pack_rows(lib, [(o, 0, None, None)], o.shape[0], o.shape[1], o.dtype, o.device, allowed)
+        if self.has_bias:
+            self.bias = torch.cat([tensors[self.names[n + "_bias"]].reshape(-1) for n in names]).contiguous()
+        if self.has_talk:
+            self.talk = tensors[self.names["talk"]].contiguous()
         if self.has_sink:
             self.sink = tensors[self.names["sink"]]
         if self.has_gate:
@@ -150,7 +188,26 @@ class Attention(Part):
             lib.head_gate(attn, logits, 0, self.n_heads, self.pad)
         return linear_to_stream(lib, attn, self.w_o, stream, next_norm)
 
+    def _forward_mixed(self, h, ctx, view, stream, next_norm):
+        """Biases, unit heads, the cache write, and attention with all heads of a token together."""
+        lib = self.env.lib
+        t, hq, hk, d = h.shape[0], self.n_heads, self.n_kv, self.pad
+        owns = self.cache_from is None
+        qkv = linear(lib, h, self.w_qkv, torch.float32)
+        q = torch.empty((t, hq, d), dtype=self.env.dtype, device=h.device)
+        lib.bias_norm_store(qkv, self.bias, self.qk_eps is not None, self.qk_eps or 0.0, q, view.k_pages if owns else None,
+                            view.v_pages if owns else None, ctx.tok_pos, ctx.tok_seq, view.block_table, hq, hk, self.head_dim,
+                            self.value_dim, d)
+        attn = torch.empty((t, hq * d), dtype=self.env.dtype, device=h.device)
+        lib.attention_mixed(q, view.k_pages, view.v_pages, attn, ctx.tok_pos, ctx.tok_seq, view.block_table, hq, hk, d,
+                            self.scale, self.talk, self.chunk or 0, int(self.window) if self.window is not None else 0)
+        return self._gate_and_project(attn, h, stream, next_norm)
+
     def forward(self, h, ctx, view, stream: Optional[torch.Tensor] = None, next_norm=None):
+        if self.mixed:
+            if hasattr(h, "tensor") and not isinstance(h, torch.Tensor):
+                h = h.tensor()
+            return self._forward_mixed(h, ctx, view, stream, next_norm)
         lib = self.env.lib
         t = h.shape[0]
         hq, hk, d = self.n_heads, self.n_kv, self.pad

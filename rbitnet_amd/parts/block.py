@@ -10,6 +10,13 @@ Who adds what to the stream, and in which form a part's output travels to the ne
 `stream.py`'s business: an arrangement calls `sublayer(part, norm, x, pending, next_norm, ...)`
 once per part and hands on what comes back.
 
+"prenorm" takes two things that a plain decoder leaves out: a layer without a feed-forward (and second norm), and a
+token shift in front of the mixer (block parameter `token_shift`: {"name": tensor}): what the mixer reads is
+    h_t + (h_(t-1) - h_t) * s      per channel, s the tensor [E], h_(t-1) the normalised row of the token before (zeros
+                                   before a sequence's first token)
+in float32; the last normalised row of a sequence is part of its state in the cache (`view.states["token_shift"]`).
+It is a causal convolution of two taps (-s on the row itself, s on the one before, added to the row), and runs as one.
+
 Interface of a block: parts() -> {name: part} for the loader (names are tensor-name
 segments below the layer's prefix); mixer (for the cache request);
 forward(x, pending, ctx, view) -> pending (a tensor still to be added, None, or GainedRows).
@@ -22,42 +29,95 @@ from typing import Dict
 
 import torch
 
-from .base import BuildEnv, build_part, register_block
+from .base import BuildEnv, Part, TensorSpec, build_part, register_block
 from ..errors import ConfigError
-from .stream import ScaledSum, normed_for, sublayer  # noqa: F401  (normed_for: its old home)
+from .short_conv import ACT_NONE, ShortConv
+from .stream import GainedRows, ScaledSum, normed_for, sublayer  # noqa: F401  (normed_for: its old home)
 
 DEFAULT_SEGMENTS = {"norm1": "input_layernorm", "mixer": "self_attn", "norm2": "post_attention_layernorm",
                     "feed_forward": "mlp"}
+
+
+class _ShiftTensor(Part):
+    """The layer's own tensor of a token shift, loaded under the layer's prefix."""
+
+    def __init__(self, block: "PreNormBlock"):
+        self.block = block
+
+    def tensor_specs(self) -> Dict[str, TensorSpec]:
+        return {self.block.shift_name: TensorSpec((self.block.hidden,), role="gain", init="normal")}
+
+    def load(self, tensors: Dict[str, torch.Tensor]) -> None:
+        s = tensors[self.block.shift_name].to(torch.float32)
+        self.block.shift.load(torch.stack([s, -s], dim=1))      # taps: the row before, the row itself
 
 
 class PreNormBlock:
     takes_next_norm = True
 
     def __init__(self, layer_spec, env: BuildEnv):
+        params = dict(getattr(layer_spec, "params", None) or {})
+        self.env, self.hidden = env, env.hidden_size
         self.norm1 = build_part("norm", layer_spec.norm1, env)
         self.mixer = build_part("mixer", layer_spec.mixer, env)
-        self.norm2 = build_part("norm", layer_spec.norm2, env)
-        self.feed_forward = build_part("feed_forward", layer_spec.feed_forward, env)
+        self.norm2 = self.feed_forward = None
+        if layer_spec.feed_forward is not None:
+            self.norm2 = build_part("norm", layer_spec.norm2, env)
+            self.feed_forward = build_part("feed_forward", layer_spec.feed_forward, env)
         self.segments = dict(DEFAULT_SEGMENTS, **(getattr(layer_spec, "segments", None) or {}))
+        shift = params.get("token_shift")
+        self.shift = ShortConv(self.hidden, 2, env, residual=True, act=ACT_NONE) if shift else None
+        self.shift_name = str(shift.get("name", "shift")) if shift else None
+        if self.shift is not None and "out_dtype" not in self.norm1.forward.__code__.co_varnames:
+            raise ConfigError("a token shift needs a norm that can leave float32 rows (rmsnorm, layernorm)")
+
+    def _all(self):
+        return [p for p in (self.norm1, self.mixer, self.norm2, self.feed_forward) if p is not None]
 
     @property
     def graph_safe(self) -> bool:
-        return all(getattr(p, "graph_safe", False) for p in (self.norm1, self.mixer, self.norm2, self.feed_forward))
+        return all(getattr(p, "graph_safe", False) for p in self._all())
 
     @property
     def plan_safe(self) -> bool:
-        return all(getattr(p, "plan_safe", False) for p in (self.norm1, self.mixer, self.norm2, self.feed_forward))
+        return all(getattr(p, "plan_safe", False) for p in self._all())
 
     def parts(self) -> Dict[str, object]:
-        return {self.segments["norm1"]: self.norm1, self.segments["mixer"]: self.mixer,
-                self.segments["norm2"]: self.norm2, self.segments["feed_forward"]: self.feed_forward}
+        out = {self.segments["norm1"]: self.norm1, self.segments["mixer"]: self.mixer}
+        if self.feed_forward is not None:
+            out[self.segments["norm2"]] = self.norm2
+            out[self.segments["feed_forward"]] = self.feed_forward
+        if self.shift is not None:
+            out[""] = _ShiftTensor(self)
+        return out
+
+    def cache_requests(self):
+        many = getattr(self.mixer, "cache_requests", None)
+        one = getattr(self.mixer, "cache_request", None)
+        out = list(many()) if many else ([one()] if one and one() is not None else [])
+        if self.shift is not None:
+            out.append(self.shift.cache_request("token_shift"))
+        return out
 
     @property
     def first_norm(self):
         return self.norm1
 
+    def _mixer(self, x: torch.Tensor, pending, after, ctx, view):
+        if self.shift is None:
+            return sublayer(self.mixer, self.norm1, x, pending, after, ctx, view)
+        # the normalised rows in float32, then the shift towards the row before, rounded once on the way out
+        delta = None if isinstance(pending, GainedRows) else pending          # such rows mean that the stream holds the sum
+        hn = self.norm1.forward(x, delta, None, out_dtype=torch.float32)
+        h = self.shift.forward(hn, ctx, view.states["token_shift"], self.env.dtype)
+        if getattr(self.mixer, "adds_to_stream", False):
+            return self.mixer.forward(h, ctx, view, stream=x, next_norm=after)
+        return self.mixer.forward(h, ctx, view)
+
     def forward(self, x: torch.Tensor, pending, ctx, view, next_norm=None):
-        a = sublayer(self.mixer, self.norm1, x, pending, self.norm2, ctx, view)
+        if self.feed_forward is None:
+            return self._mixer(x, pending, next_norm, ctx, view)
+        a = self._mixer(x, pending, self.norm2, ctx, view)
         return sublayer(self.feed_forward, self.norm2, x, a, next_norm, ctx)
 
 

@@ -8,14 +8,17 @@ Their tensors have no layer prefix: `tensor_specs` names them in full.
 
 embedding "table" (crates/bitnet-core/src/llama/model.rs:229-232): x[t, :] = table[id[t], :].
     Parameters: name, vocab_size, streams (None: the stream is [T, E]; n: n equal copies [n, T, E], for
-    blocks that keep the residual stream in several copies).
+    blocks that keep the residual stream in several copies), scale (None, or c: the rows are multiplied by c),
+    positions (None, or {"name": tensor, "max_positions": n}: a learned vector per absolute position [n, E], added
+    to the scaled row as it is): x[t, :] = table[id[t], :] * c + positions[pos[t], :].
     Interface of an embedding: tensor_specs() / load(tensors) / forward(ctx) -> float32 [T, E]
     (ctx.token_ids int32 [T]); `table` if a head may share it.
 
 head "linear" (model.rs:309-315): logits = W norm(x), on the asked rows only; W is the
     embedding's table when the parameters name no matrix (tied).
     Parameters: norm (a PartSpec), norm_name, name (None: tied), vocab_size, softcap (None, or c:
-    logits <- c tanh(logits / c)).  A stream in several copies is summed by the norm.
+    logits <- c tanh(logits / c)), logit_scale (None, or s: logits <- s logits, before a cap).  A stream in several
+    copies is summed by the norm.
     Interface of a head: tensor_specs() / load(tensors, embedding) /
     forward(x, pending, rows, ctx) -> float32 [len(rows), V], where x is the stream, `pending`
     what the last block left to be added (see stream.py) and rows the packed rows asked for;
@@ -45,13 +48,25 @@ class TableEmbedding(Part):
         self.vocab_size = int(params["vocab_size"])
         self.hidden = env.hidden_size
         self.streams = None if params.get("streams") is None else int(params["streams"])
+        self.scale = None if params.get("scale") is None else float(params["scale"])
+        pos = params.get("positions")
+        self.pos_name = None if pos is None else str(pos["name"])
+        self.max_positions = None if pos is None else int(pos["max_positions"])
+        if (self.scale is not None or pos is not None) and self.streams is not None:
+            raise ConfigError("an embedding with a scale or learned positions fills one copy of the stream")
         self.table: Optional[torch.Tensor] = None
+        self.positions: Optional[torch.Tensor] = None
 
     def tensor_specs(self) -> Dict[str, TensorSpec]:
-        return {self.name: TensorSpec((self.vocab_size, self.hidden))}
+        out = {self.name: TensorSpec((self.vocab_size, self.hidden))}
+        if self.pos_name is not None:
+            out[self.pos_name] = TensorSpec((self.max_positions, self.hidden))
+        return out
 
     def load(self, tensors: Dict[str, torch.Tensor]) -> None:
         self.table = tensors[self.name]
+        if self.pos_name is not None:
+            self.positions = tensors[self.pos_name]
 
     def step_bytes(self, element_size: int) -> int:
         return 0                      # the gather reads a few rows only
@@ -62,7 +77,11 @@ class TableEmbedding(Part):
             self.env.lib.embed_streams(self.table, ctx.token_ids, x)
             return x
         x = torch.empty((ctx.n_tokens, self.hidden), dtype=torch.float32, device=self.table.device)
-        self.env.lib.embed_gather(self.table, ctx.token_ids, x)
+        if self.scale is not None or self.positions is not None:
+            self.env.lib.embed_scaled_pos(self.table, ctx.token_ids, 1.0 if self.scale is None else self.scale,
+                                          self.positions, ctx.tok_pos, x)
+        else:
+            self.env.lib.embed_gather(self.table, ctx.token_ids, x)
         return x
 
 
@@ -79,6 +98,7 @@ class LinearHead(Part):
         self.softcap = None if params.get("softcap") is None else float(params["softcap"])
         if self.softcap is not None and not self.softcap > 0:
             raise ConfigError(f"a head's softcap must be positive, found {self.softcap}")
+        self.logit_scale = None if params.get("logit_scale") is None else float(params["logit_scale"])
         self.weight = None
 
     @property
@@ -129,6 +149,8 @@ class LinearHead(Part):
     def forward(self, x: torch.Tensor, pending, rows: torch.Tensor, ctx=None) -> torch.Tensor:
         xn = normed_for(self, self.norm, x, pending, rows)
         logits = linear(self.env.lib, xn, self.weight, torch.float32)
+        if self.logit_scale is not None:
+            self.env.lib.scale(logits, self.logit_scale)
         if self.softcap is not None:
             self.env.lib.tanh_cap(logits, self.softcap)
         return logits

@@ -59,22 +59,30 @@ class SwiGLU(Part):
         return linear_to_stream(lib, t, self.w_down, stream, next_norm)
 
 
-class DenseXielu(Part):
-    """out = Wdown act(Wup h) with act = xIELU: for z > 0, softplus(p) z^2 + z / 2; for z <= 0,
-    (1/2 + softplus(q)) (exp(z) - 1 - z) + z / 2, (p, q) being the two numbers of the tensor `act`.
-    Parameters: intermediate_size, names ({"up", "down", "act"})."""
+class DenseAct(Part):
+    """out = Wdown act(Wup h), the activation applied where the first product stores its float32 sums.
+    activation "xielu": for z > 0, softplus(p) z^2 + z / 2; for z <= 0, (1/2 + softplus(q)) (exp(z) - 1 - z) + z / 2,
+    (p, q) being the two numbers of the tensor `act`.  activation "gelu_tanh": z / 2 (1 + tanh(sqrt(2 / pi) (z + 0.044715 z^3))),
+    no tensor.  Parameters: intermediate_size, activation, names ({"up", "down", "act"})."""
     graph_safe = True
     plan_safe = True
+    adds_to_stream = True
+    activation = "xielu"
 
     def __init__(self, params: Dict, env: BuildEnv):
         self.env = env
         self.ff = int(params["intermediate_size"])
+        self.activation = str(params.get("activation", type(self).activation))
+        if self.activation not in ("xielu", "gelu_tanh"):
+            raise ConfigError(f"dense feed-forward: activation {self.activation!r} not supported (xielu, gelu_tanh)")
         self.names = dict({"up": "up", "down": "down", "act": "act"}, **(params.get("names") or {}))
         self.hidden = env.hidden_size
 
     def tensor_specs(self) -> Dict[str, TensorSpec]:
-        return {self.names["up"]: TensorSpec((self.ff, self.hidden)), self.names["down"]: TensorSpec((self.hidden, self.ff)),
-                self.names["act"]: TensorSpec((2,), role="gain", init="normal")}
+        out = {self.names["up"]: TensorSpec((self.ff, self.hidden)), self.names["down"]: TensorSpec((self.hidden, self.ff))}
+        if self.activation == "xielu":
+            out[self.names["act"]] = TensorSpec((2,), role="gain", init="normal")
+        return out
 
     def load(self, tensors: Dict[str, torch.Tensor]) -> None:
         allowed = not getattr(self.env, "generic_only", False)
@@ -82,13 +90,26 @@ class DenseXielu(Part):
         self.w_up = pack_rows(self.env.lib, [(up, 0, None, None)], up.shape[0], up.shape[1], up.dtype, up.device, allowed)
         self.w_down = pack_rows(self.env.lib, [(down, 0, None, None)], down.shape[0], down.shape[1], down.dtype,
                                 down.device, allowed)
-        self.act = tensors[self.names["act"]]
+        if self.activation == "xielu":
+            self.act = tensors[self.names["act"]]
+        else:       # the kernels read a first number that is no number as "the tanh form of GELU"
+            self.act = torch.tensor([float("nan"), 0.0], dtype=torch.float32, device=up.device)
 
     def forward(self, h, ctx=None, stream: Optional[torch.Tensor] = None, next_norm=None):
         lib = self.env.lib
         t = xielu_linear(lib, h, self.w_up, self.act, self.env.dtype)      # the activation in the product's epilogue
-        return linear(lib, t, self.w_down, torch.float32)
+        return linear_to_stream(lib, t, self.w_down, stream, next_norm)
+
+
+class DenseXielu(DenseAct):
+    activation = "xielu"
+
+
+class DenseGelu(DenseAct):
+    activation = "gelu_tanh"
 
 
 register_feed_forward("swiglu", SwiGLU)
 register_feed_forward("dense_xielu", DenseXielu)
+register_feed_forward("dense_gelu", DenseGelu)
+register_feed_forward("dense_act", DenseAct)

@@ -28,6 +28,10 @@ from .stream import GainedRows, ScaledSum, StreamsUpdate  # noqa: F401  (GainedR
 
 
 class RMSNorm(Part):
+    """Parameters: size, eps, and two that a plain decoder leaves out: scalar (True: the gain is ONE number for all
+    coordinates, a tensor without dimensions; it is spread over the width at load time, so that every kernel and every
+    folding of the norm into products serves as it is), names ({"weight": ...}: the tensor's name below the part's prefix;
+    an empty name is the prefix itself)."""
     graph_safe = True
     plan_safe = True
     folds_into_products = True
@@ -36,19 +40,26 @@ class RMSNorm(Part):
     def __init__(self, params: Dict, env: BuildEnv):
         self.size = int(params["size"])
         self.eps = float(params["eps"])
+        self.scalar = bool(params.get("scalar", False))
+        self.names = dict({"weight": "weight"}, **(params.get("names") or {}))
         self.env = env
         self.weight: Optional[torch.Tensor] = None
 
     def tensor_specs(self) -> Dict[str, TensorSpec]:
-        return {"weight": TensorSpec((self.size,), role="gain", init="ones_normal")}
+        return {self.names["weight"]: TensorSpec(() if self.scalar else (self.size,), role="gain", init="ones_normal")}
+
+    def tensor_names(self, base: str) -> Dict[str, str]:
+        """full name -> the part's own name, for an owner that stores the norm under `base`."""
+        return {".".join(p for p in (base, name) if p): name for name in self.tensor_specs()}
 
     def load(self, tensors: Dict[str, torch.Tensor]) -> None:
-        self.weight = tensors["weight"]
+        w = tensors[self.names["weight"]]
+        self.weight = w.reshape(1).expand(self.size).contiguous() if self.scalar else w
 
     def forward(self, x: torch.Tensor, delta: Optional[torch.Tensor] = None,
-                rows: Optional[torch.Tensor] = None) -> torch.Tensor:
+                rows: Optional[torch.Tensor] = None, out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
         n = x.shape[0] if rows is None else rows.shape[0]
-        out = torch.empty((n, self.size), dtype=self.env.dtype, device=x.device)
+        out = torch.empty((n, self.size), dtype=out_dtype or self.env.dtype, device=x.device)
         self.env.lib.add_rmsnorm(x, delta, self.weight, self.eps, rows, out)
         return out
 
