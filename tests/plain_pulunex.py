@@ -65,7 +65,8 @@ def attention_keys_values(h: torch.Tensor, w: Dict[str, torch.Tensor], m: Dict, 
     return unit_rms(k, eps), v
 
 
-def talking_attention(h: torch.Tensor, w: Dict[str, torch.Tensor], m: Dict, eps: float, k: torch.Tensor, v: torch.Tensor):
+def mixed_weights(h: torch.Tensor, w: Dict[str, torch.Tensor], m: Dict, eps: float, k: torch.Tensor) -> torch.Tensor:
+    """the softmax weights [H, T, T] of every head: zero where a key is not seen"""
     t, hq, g, d = h.shape[0], m["heads"], m["kv_heads"], m["dim"]
     q = unit_rms((h @ w["q"].to(F64).T + w["q.b"].to(F64)).view(t, hq, d).transpose(0, 1), eps)       # [H, T, d]
     kv_of = torch.arange(hq) // (hq // g)
@@ -73,7 +74,13 @@ def talking_attention(h: torch.Tensor, w: Dict[str, torch.Tensor], m: Dict, eps:
     b = torch.einsum("hg,gij->hij", w["talk"].to(F64), a)
     chunk = (m.get("mask") or {}).get("size")
     b = b.masked_fill(~visible(t, chunk)[None], -math.inf)
-    p = torch.softmax(b, dim=-1)
+    return torch.softmax(b, dim=-1)
+
+
+def talking_attention(h: torch.Tensor, w: Dict[str, torch.Tensor], m: Dict, eps: float, k: torch.Tensor, v: torch.Tensor):
+    t, hq, g = h.shape[0], m["heads"], m["kv_heads"]
+    p = mixed_weights(h, w, m, eps, k)
+    kv_of = torch.arange(hq) // (hq // g)
     o = torch.einsum("hij,hje->ihe", p, v[kv_of]).reshape(t, hq * m["vdim"])
     return o @ w["o"].to(F64).T
 
@@ -143,6 +150,14 @@ def forward(config: Dict, tensors: Dict[str, torch.Tensor], ids, streams: Option
             streams.append(x.clone())
     xn = scalar_rmsnorm(x, tensors["final.norm"], eps)
     return xn @ tensors["head"].to(F64).T * float(config["logit_scale"])
+
+
+class PlainPulunex:
+    def __init__(self, config: Dict, tensors: Dict[str, torch.Tensor]):
+        self.config, self.tensors = config, tensors
+
+    def logits(self, ids, streams: Optional[list] = None) -> torch.Tensor:
+        return forward(self.config, self.tensors, ids, streams)
 
 
 # ---------------------------------------------------------------------- random models for the tests
