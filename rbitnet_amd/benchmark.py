@@ -358,8 +358,30 @@ def tigutar_config(width: int, layers: int, heads: int, kv_heads: int, ff: int, 
     return {"architecture": "Tigutar", "vocab": vocab, "width": width, "residual_mult": 0.5, "norm": {"eps": 1e-5}, "layers": out}
 
 
-# size -> (the design's configuration, the Llama shape of equal width, depth and feed-forward width beside it)
+def pulunex_config(width: int, layers: int, heads: int, kv_heads: int, ff: int, vocab: int, experts: int = 16, top: int = 4,
+                   identity: int = 2, chunk: int = 1024, dim: int = 64, max_positions: int = 8192) -> dict:
+    """Attention with mixed heads in chunks: the first layer has a dense feed-forward, the others routed experts whose
+    `top` chosen ones are together as wide as the dense one, beside a shared expert of an eighth of it; the layers of the
+    second half read the keys and values of the last layer of the first half."""
+    mixer = {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": dim, "scale": 8.0 / dim, "mask": {"size": chunk}}
+    moe = {"kind": "moe", "expert": {"ff": ff // top}, "router": {"experts": experts, "top": top, "identity": identity},
+           "shared": {"ff": ff // 8}}
+    out, keeper = [], layers // 2 - 1
+    for i in range(layers):
+        m = dict(mixer, kv_from=keeper) if i > keeper >= 0 else dict(mixer)
+        out.append({"type": "attention", "mixer": m, "mlp": {"kind": "dense", "ff": ff} if i == 0 else moe})
+    return {"architecture": "Pulunex", "vocab": vocab, "width": width, "max_positions": max_positions, "embedding": {"scale": 2.0},
+            "logit_scale": 0.5, "norm": {"eps": 1e-5}, "layers": out}
+
+
+# size -> (the design's configuration, then the shapes beside it: the Llama shape of equal width, depth and feed-forward
+# width, and for Pulunex the Tigutar model of those sizes too, whose routed experts and attention kernels are the like ones)
 DESIGN_SIZES = {
+    "pulunex_w1024": (pulunex_config(1024, 12, 16, 4, 4096, 32000), tigutar_config(1024, 12, 16, 4, 4096, 32000, experts=16),
+                      _other(1024, 4096, 16, 4, 64, 12, vocab=32000)),
+    "pulunex_w2048": (pulunex_config(2048, 16, 32, 8, 8192, 128256), tigutar_config(2048, 16, 32, 8, 8192, 128256, experts=16),
+                      _other(2048, 8192, 32, 8, 64, 16)),
+    "pulunex_w4096": (pulunex_config(4096, 8, 32, 8, 14336, 128256, dim=128), dict(LLAMA3_8B, num_hidden_layers=8)),
     "tigutar_w1024": (tigutar_config(1024, 12, 16, 4, 4096, 32000, experts=16), _other(1024, 4096, 16, 4, 64, 12, vocab=32000)),
     "tigutar_w2048": (tigutar_config(2048, 16, 32, 8, 8192, 128256), _other(2048, 8192, 32, 8, 64, 16)),
     "tigutar_w4096": (tigutar_config(4096, 8, 64, 16, 14336, 128256), dict(LLAMA3_8B, num_hidden_layers=8)),
@@ -403,8 +425,9 @@ def design_run(size: str, dtype: str, batch: int, steps: int, warmup: int, prefi
         cfg = dict(cfg)
         label = "llama" if "architectures" in cfg else str(cfg["architecture"]).lower()
         ctx_cap = prompt_len + steps + warmup + 64
-        if "max_position_embeddings" in cfg:
-            cfg["max_position_embeddings"] = max(cfg["max_position_embeddings"], prefill_tokens + 64, ctx_cap)
+        for key in ("max_position_embeddings", "max_positions"):
+            if key in cfg:
+                cfg[key] = max(cfg[key], prefill_tokens + 64, ctx_cap)
         engine = Engine.random(cfg, seed=0, dtype="bfloat16" if dtype == "bf16" else "float32", std=0.02, norm_std=0.02,
                                max_batch=batch, max_tokens=max(batch * ctx_cap, prefill_tokens + 64),
                                max_seq_len=max(ctx_cap, prefill_tokens + 64))
@@ -479,8 +502,8 @@ def main(argv=None) -> int:
                     help="no benchmark line: the named shape's decode products of 8 tokens beside a kernel that only "
                          "reads as many bytes")
     ap.add_argument("--design", default="", metavar="SIZE",
-                    help=f"no benchmark line: a Bagonex or Tigutar model of this size ({', '.join(sorted(DESIGN_SIZES))}) beside the Llama "
-                         "shape of equal width, depth and feed-forward width: prefill and decode throughput, and the time per kernel")
+                    help=f"no benchmark line: a Bagonex, Tigutar or Pulunex model of this size ({', '.join(sorted(DESIGN_SIZES))}) beside the Llama "
+                         "shape of equal width, depth and feed-forward width (Pulunex: beside Tigutar too): prefill and decode throughput, and the time per kernel")
     ap.add_argument("--tokens", default="1,8,64,512,2048", help="token counts of --planner-sweep")
     ap.add_argument("--sweep-detail", default=None, help="--planner-sweep: a file for every candidate's time")
     ap.add_argument("--prefill-tokens", type=int, default=PREFILL_TOKENS,

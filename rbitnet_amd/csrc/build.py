@@ -26,7 +26,7 @@ LIB_NAME = "librbitnet_hip.so"
 ARCH = "gfx950"
 SOURCES = ["elementwise.hip", "gemm_generic.hip", "gemm_mfma.hip", "gemm_skinny.hip", "gemm_tiled.hip",
            "attention_generic.hip", "attention_mfma.hip", "sampling.hip", "weights_init.hip", "probe.hip", "plan.hip", "streams.hip", "recurrent.hip",
-           "latent.hip", "mixers.hip", "routed.hip", "talking.hip"]
+           "latent.hip", "mixers.hip", "routed.hip", "talking.hip", "talking_mfma.hip"]
 HEADERS = ["api.h", "tune.h", "common.h", "mfma.h", "gemm_internal.h"]
 FLAGS = ["-O3", "-std=c++17", "-fPIC", f"--offload-arch={ARCH}", "-Xclang", "-target-feature", "-Xclang",
          "-packed-fp32-ops", "-Wno-unused-result", "-Wno-unknown-warning-option"]

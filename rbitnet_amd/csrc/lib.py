@@ -105,7 +105,7 @@ class KernelTimes:
         return "\n".join(lines)
 
 
-TIMED_OPS = ("route_choose", "experts_combine", "embed_scaled_pos", "scale", "bias_norm_store", "attention_mixed", "recurrence_prep", "linear_recurrence", "layernorm_residual", "rope_store", "head_gate", "pair_norm_mean",
+TIMED_OPS = ("route_choose", "experts_combine", "embed_scaled_pos", "scale", "bias_norm_store", "attention_mixed", "attention_mixed_bf16", "recurrence_prep", "linear_recurrence", "layernorm_residual", "rope_store", "head_gate", "pair_norm_mean",
              "route_top", "routed_experts", "pairs_sum", "embed_streams", "streams_layernorm", "streams_update", "xielu", "tanh_cap", "short_conv",
              "delta_prep", "delta_rule", "gated_rmsnorm", "latent_norm_store", "heads_linear", "attention_sinks", "embed_gather", "add_rmsnorm", "rope_kv_write", "swiglu", "gemm_generic", "gemm_bf16", "gemm_bf16_terms",
              "gemm_bf16_few", "attention_generic", "attention_prefill_bf16", "attention_decode_bf16",
@@ -182,6 +182,7 @@ class Kernels:
             "rb_scale": [_P, _F, _L, _P],
             "rb_bias_norm_store": [_P, _L, _P, _I, _F, _P, _P, _P, _I, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _P],
             "rb_attention_mixed": [_P, _P, _P, _P, _I, _P, _P, _P, _I, _I, _I, _I, _I, _F, _P, _I, _I, _P],
+            "rb_attention_mixed_bf16": [_P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _P, _I, _I, _P],
         }
         for name, args in sig.items():
             fn = getattr(L, name)
@@ -905,6 +906,32 @@ class Kernels:
         self._ok(self._lib.rb_attention_mixed(_ptr(q), _ptr(k_pages), _ptr(v_pages), _ptr(out), dtype_code(q.dtype), _ptr(tok_pos),
                                               _ptr(tok_seq), _ptr(block_table), block_table.shape[1], n, n_heads, n_kv, head_dim,
                                               float(scale), _ptr(talk), int(chunk or 0), int(window or 0), self._stream()))
+
+    def attention_mixed_bf16(self, q, k_pages, v_pages, out, ctx, block_table, n_heads, n_kv, head_dim, scale, talk, chunk,
+                             window) -> None:
+        """attention_mixed on the matrix cores: bfloat16, head_dim 64 or 128, at most 32 heads; the step's sequences from
+        ctx (cu_seqlens, past_len)."""
+        n = q.shape[0]
+        _check(q, "q", torch.bfloat16, (n, n_heads, head_dim))
+        _check(k_pages, "k_pages", torch.bfloat16)
+        _check(v_pages, "v_pages", torch.bfloat16, k_pages.shape)
+        if tuple(k_pages.shape[1:]) != (n_kv, self.page_size, head_dim):
+            raise KernelError("cache pages do not match the head counts")
+        if head_dim not in (64, 128) or n_heads > 32 or n_heads % n_kv:
+            raise KernelError(f"attention_mixed_bf16: {n_heads} heads of {head_dim} numbers not supported (64 or 128, at most 32 heads)")
+        if n != ctx.n_tokens:
+            raise KernelError(f"attention_mixed_bf16: {n} rows for a step of {ctx.n_tokens} tokens")
+        _check(out, "out", torch.bfloat16, (n, n_heads * head_dim))
+        _check(ctx.cu_seqlens, "cu_seqlens", torch.int32, (ctx.n_seqs + 1,))
+        _check(ctx.past_len, "past_len", torch.int32, (ctx.n_seqs,))
+        _check(block_table, "block_table", torch.int32)
+        if block_table.shape[0] < ctx.n_seqs:
+            raise KernelError("attention_mixed_bf16: the block table has fewer rows than the step has sequences")
+        _check(talk, "talk", torch.float32, (n_heads, n_heads))
+        self._ok(self._lib.rb_attention_mixed_bf16(_ptr(q), _ptr(k_pages), _ptr(v_pages), _ptr(out), _ptr(ctx.cu_seqlens),
+                                                   _ptr(ctx.past_len), _ptr(block_table), block_table.shape[1], ctx.n_seqs, n,
+                                                   n_heads, n_kv, head_dim, float(scale), _ptr(talk), int(chunk or 0),
+                                                   int(window or 0), self._stream()))
 
     def pairs_sum(self, pairs: torch.Tensor, top: int, out: torch.Tensor) -> None:
         n, width = out.shape

@@ -58,6 +58,7 @@ from .linear import linear, linear_or_terms, linear_to_stream, pack_rows
 DEFAULT_NAMES = {"q": "q_proj.weight", "k": "k_proj.weight", "v": "v_proj.weight", "o": "o_proj.weight", "sink": "sink",
                  "gate": "gate", "q_bias": "q_proj.bias", "k_bias": "k_proj.bias", "v_bias": "v_proj.bias", "talk": "talk"}
 MIXED_MAX_HEADS, MIXED_MAX_NUMBERS = 64, 8192      # what the kernels that take all heads of a token together hold
+MIXED_MATRIX_CORE_HEADS = 32                       # and the one on the matrix cores
 _MATRIX_CORE_HEAD_DIMS = (64, 128)
 _DECODE_GROUPS = tuple(range(1, 17))    # query heads per kv head the decode kernels take
 
@@ -115,6 +116,7 @@ class Attention(Part):
                                   f"heads of a token together hold ({MIXED_MAX_HEADS} heads, {MIXED_MAX_NUMBERS} numbers)")
         self.bias: Optional[torch.Tensor] = None
         self.talk: Optional[torch.Tensor] = None
+        self.mixed_on_matrix_cores = False
         self.w_gate = None
         self.sink: Optional[torch.Tensor] = None
         self.w_qkv: Optional[torch.Tensor] = None
@@ -164,6 +166,11 @@ class Attention(Part):
             self.bias = torch.cat([tensors[self.names[n + "_bias"]].reshape(-1) for n in names]).contiguous()
         if self.has_talk:
             self.talk = tensors[self.names["talk"]].contiguous()
+        # the matrix cores' kernel: bfloat16, heads of 64 or 128 numbers, at most 32 of them; it wants a mixing matrix
+        self.mixed_on_matrix_cores = bool(self.mixed and allowed and self.env.dtype == torch.bfloat16
+                                          and self.pad in _MATRIX_CORE_HEAD_DIMS and self.n_heads <= MIXED_MATRIX_CORE_HEADS)
+        if self.mixed_on_matrix_cores and self.talk is None:
+            self.talk = torch.eye(self.n_heads, dtype=torch.float32, device=o.device)
         if self.has_sink:
             self.sink = tensors[self.names["sink"]]
         if self.has_gate:
@@ -199,8 +206,13 @@ class Attention(Part):
                             view.v_pages if owns else None, ctx.tok_pos, ctx.tok_seq, view.block_table, hq, hk, self.head_dim,
                             self.value_dim, d)
         attn = torch.empty((t, hq * d), dtype=self.env.dtype, device=h.device)
-        lib.attention_mixed(q, view.k_pages, view.v_pages, attn, ctx.tok_pos, ctx.tok_seq, view.block_table, hq, hk, d,
-                            self.scale, self.talk, self.chunk or 0, int(self.window) if self.window is not None else 0)
+        window = int(self.window) if self.window is not None else 0
+        if self.mixed_on_matrix_cores:
+            lib.attention_mixed_bf16(q, view.k_pages, view.v_pages, attn, ctx, view.block_table, hq, hk, d, self.scale, self.talk,
+                                     self.chunk or 0, window)
+        else:
+            lib.attention_mixed(q, view.k_pages, view.v_pages, attn, ctx.tok_pos, ctx.tok_seq, view.block_table, hq, hk, d,
+                                self.scale, self.talk, self.chunk or 0, window)
         return self._gate_and_project(attn, h, stream, next_norm)
 
     def forward(self, h, ctx, view, stream: Optional[torch.Tensor] = None, next_norm=None):

@@ -200,7 +200,7 @@ def save_file(path: str, tensors: Iterable[Tuple[str, torch.Tensor]], metadata: 
             if t.dtype != dtype or tuple(t.shape) != tuple(shape):
                 raise WeightError(f"tensor {name!r} does not match the announced layout")
             t = t.detach().to("cpu").contiguous()
-            f.write(t.view(torch.uint8).numpy().tobytes() if t.numel() else b"")
+            f.write(t.reshape(-1).view(torch.uint8).numpy().tobytes() if t.numel() else b"")      # reshape: a tensor without dimensions
             written.append(name)
         if written != list(layout):
             raise WeightError("tensors were not written in the announced order")
