@@ -4,13 +4,16 @@
 // A workgroup of 4 waves takes 16 consecutive queries of one sequence and ALL heads, since every head's weights need
 // every head's scores.  The keys go by in tiles of 64 (a page).  Per tile:
 //   1. scores      S[g, i, j] = q_gi . k_j * scale for every head g: bfloat16 MFMA 16x16x32, operands straight from memory
-//                  (a query's and a key's 8 numbers are 16 bytes in a row); float32 into LDS, zero where j is not seen
+//                  (a query's and a key's 8 numbers are 16 bytes in a row); a wave takes a quarter of the heads, keeps
+//                  their queries in registers for all tiles where they fit, and asks for a kv head's 64 keys at once;
+//                  float32 into LDS, zero where j is not seen
 //   2. mixing      S[h, i, j] <- sum_g talk[h, g] S[g, i, j]: float32 MFMA 16x16x4 (float32 inputs and sums), talk in
 //                  registers, 16 (i, j) columns at a time, in place
 //   3. softmax     online, per (h, i) row in float32; the weights leave as TWO bfloat16 numbers (p = hi + lo, which holds
 //                  16 bits of p), written over the row's scores
 //   4. values      per kv head: V^T of the tile through LDS, O_h += P_hi V + P_lo V (bfloat16 MFMA, float32 sums); a wave
-//                  owns 16 (or 32) of a head's output numbers for all heads
+//                  owns 16 (or 32) of a head's output numbers for all heads; the next kv head's (or tile's) values are on
+//                  their way from memory while the products of this one run
 // What a row has seen so far (maximum, sum) lives in registers of the wave that does the row's softmax.
 #include <math.h>
 
@@ -99,36 +102,90 @@ __global__ __launch_bounds__(TM_THREADS) void attention_mixed_mfma_kernel(
 #pragma unroll
     for (int d = 0; d < DB; ++d) oacc[h][d] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 
-  // the query row this lane feeds into the score MFMAs (rows past the sequence's end read its last row)
+  // ---- the heads whose scores this wave computes, and their queries (rows past the sequence's end read its last row)
+  constexpr bool QR = HW * (D / 32) <= 16;      // the queries stay in registers
+  const int hpw = (n_heads + 3) / 4;
+  const int h_lo = wave * hpw, h_hi = h_lo + hpw < n_heads ? h_lo + hpw : n_heads;
   const size_t q_row = ((size_t)(seq_start + q0 + (l16 < n_valid ? l16 : n_valid - 1)) * n_heads) * D + lg * 8;
+  Frag8 qres[QR ? HW * (D / 32) : 1];
+  if (QR) {
+#pragma unroll
+    for (int k = 0; k < HW; ++k)
+#pragma unroll
+      for (int s = 0; s < D / 32; ++s)
+        qres[k * (D / 32) + s].u = h_lo + k < h_hi ? load16(q + q_row + (size_t)(h_lo + k) * D + s * 32) : zero16();
+  }
+
+  // ---- V^T of a tile and kv head: a thread takes 4 keys in a row and 8 numbers of each, and writes 8 times 4 keys
+  const int v_kq = tid & 15, v_dc = tid >> 4;
+  const bool v_on = tid < 16 * (D / 8);
+  uint4 vreg[4];
+  auto load_v = [&](int kt, int g) {
+    if (!v_on) return;
+    const bf16_t* src = v_pages + ((size_t)bt[kt] * n_kv + g) * RB_PAGE * D + (size_t)(4 * v_kq) * D + v_dc * 8;
+#pragma unroll
+    for (int e = 0; e < 4; ++e)      // what lies beyond the sequence may be anything, even NaN: zeros
+      vreg[e] = kt * RB_PAGE + 4 * v_kq + e <= kv_last ? load16(src + (size_t)e * D) : zero16();
+  };
+  auto store_v = [&]() {
+    if (!v_on) return;
+    const uint32_t w[4][4] = {{vreg[0].x, vreg[1].x, vreg[2].x, vreg[3].x}, {vreg[0].y, vreg[1].y, vreg[2].y, vreg[3].y},
+                              {vreg[0].z, vreg[1].z, vreg[2].z, vreg[3].z}, {vreg[0].w, vreg[1].w, vreg[2].w, vreg[3].w}};
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+      uint2 even, odd;
+      even.x = (w[c][0] & 0xffffu) | (w[c][1] << 16);
+      even.y = (w[c][2] & 0xffffu) | (w[c][3] << 16);
+      odd.x = (w[c][0] >> 16) | (w[c][1] & 0xffff0000u);
+      odd.y = (w[c][2] >> 16) | (w[c][3] & 0xffff0000u);
+      *reinterpret_cast<uint2*>(vt + (v_dc * 8 + 2 * c) * TM_VLD + 4 * v_kq) = even;
+      *reinterpret_cast<uint2*>(vt + (v_dc * 8 + 2 * c + 1) * TM_VLD + 4 * v_kq) = odd;
+    }
+  };
+  load_v(first_tile, 0);
 
   for (int kt = first_tile; kt <= last_tile; ++kt) {
     const size_t page_base = (size_t)bt[kt] * n_kv * RB_PAGE * D;
     const int key0 = kt * RB_PAGE;
     // ---------------------------------------------------------------- 1. scores
-    for (int item = wave; item < n_kv * 4; item += 4) {
-      const int g = item >> 2, kb = item & 3;
-      const bf16_t* krow = k_pages + page_base + ((size_t)g * RB_PAGE + kb * 16 + l16) * D + lg * 8;
-      Frag8 kf[D / 32];
+    {
+      Frag8 kf[4][D / 32];
+      int g_have = -1;
 #pragma unroll
-      for (int s = 0; s < D / 32; ++s) kf[s].u = load16(krow + s * 32);
-      const int key = key0 + kb * 16 + l16;
-      for (int hh = 0; hh < group; ++hh) {
-        const int h = g * group + hh;
-        const bf16_t* qr = q + q_row + (size_t)h * D;
-        f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
+      for (int k = 0; k < HW; ++k) {
+        const int h = h_lo + k;
+        if (h < h_hi) {
+          const int g = h / group;
+          if (g != g_have) {           // the 64 keys of this kv head, asked for together
+            const bf16_t* krow = k_pages + page_base + ((size_t)g * RB_PAGE + l16) * D + lg * 8;
 #pragma unroll
-        for (int s = 0; s < D / 32; ++s) {
-          Frag8 qf;
-          qf.u = load16(qr + s * 32);
-          acc = mfma16(qf, kf[s], acc);
-        }
-        float* dst = S + (size_t)h * TM_HEAD + kb * 16 + l16;
+            for (int kb = 0; kb < 4; ++kb)
 #pragma unroll
-        for (int r = 0; r < 4; ++r) {
-          const int i = 4 * lg + r;
-          const bool seen = i < n_valid && key <= pos_first + i && key >= lo_r[r];
-          dst[i * TM_ROW] = seen ? acc[r] * scale : 0.f;       // a select: what lies beyond the sequence may be anything
+              for (int s = 0; s < D / 32; ++s) kf[kb][s].u = load16(krow + (size_t)kb * 16 * D + s * 32);
+            g_have = g;
+          }
+          Frag8 qf[D / 32];
+#pragma unroll
+          for (int s = 0; s < D / 32; ++s) {
+            if (QR)
+              qf[s] = qres[k * (D / 32) + s];
+            else
+              qf[s].u = load16(q + q_row + (size_t)h * D + s * 32);
+          }
+          float* dst = S + (size_t)h * TM_HEAD + l16;
+#pragma unroll
+          for (int kb = 0; kb < 4; ++kb) {
+            f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int s = 0; s < D / 32; ++s) acc = mfma16(qf[s], kf[kb][s], acc);
+            const int key = key0 + kb * 16 + l16;
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+              const int i = 4 * lg + r;
+              const bool seen = i < n_valid && key <= pos_first + i && key >= lo_r[r];
+              dst[i * TM_ROW + kb * 16] = seen ? acc[r] * scale : 0.f;       // a select: a key beyond the sequence may be anything
+            }
+          }
         }
       }
     }
@@ -218,28 +275,11 @@ __global__ __launch_bounds__(TM_THREADS) void attention_mixed_mfma_kernel(
     __syncthreads();
     // ---------------------------------------------------------------- 4. values, one kv head after the other
     for (int g = 0; g < n_kv; ++g) {
-      // V^T of the tile: a thread takes 4 keys in a row and 8 numbers of each, and writes 8 times 4 keys
-      if (tid < 16 * (D / 8)) {
-        const int kq = tid & 15, dc = tid >> 4;
-        uint4 vreg[4];
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          const int key = key0 + 4 * kq + e;
-          vreg[e] = key <= kv_last ? load16(v_pages + page_base + ((size_t)g * RB_PAGE + 4 * kq + e) * D + dc * 8) : zero16();
-        }
-        const uint32_t w[4][4] = {{vreg[0].x, vreg[1].x, vreg[2].x, vreg[3].x}, {vreg[0].y, vreg[1].y, vreg[2].y, vreg[3].y},
-                                  {vreg[0].z, vreg[1].z, vreg[2].z, vreg[3].z}, {vreg[0].w, vreg[1].w, vreg[2].w, vreg[3].w}};
-#pragma unroll
-        for (int c = 0; c < 4; ++c) {
-          uint2 even, odd;
-          even.x = (w[c][0] & 0xffffu) | (w[c][1] << 16);
-          even.y = (w[c][2] & 0xffffu) | (w[c][3] << 16);
-          odd.x = (w[c][0] >> 16) | (w[c][1] & 0xffff0000u);
-          odd.y = (w[c][2] >> 16) | (w[c][3] & 0xffff0000u);
-          *reinterpret_cast<uint2*>(vt + (dc * 8 + 2 * c) * TM_VLD + 4 * kq) = even;
-          *reinterpret_cast<uint2*>(vt + (dc * 8 + 2 * c + 1) * TM_VLD + 4 * kq) = odd;
-        }
-      }
+      store_v();
+      if (g + 1 < n_kv)
+        load_v(kt, g + 1);
+      else if (kt < last_tile)
+        load_v(kt + 1, 0);
       __syncthreads();
 #pragma unroll
       for (int h = 0; h < HB; ++h) {
