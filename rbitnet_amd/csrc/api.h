@@ -281,10 +281,12 @@ int rb_attention_mixed(const void* q, const void* k_pages, const void* v_pages, 
                        int n_kv_heads, int head_dim, float scale, const float* talk, int chunk, int window, void* stream);
 // The same on the matrix cores: bfloat16, head_dim 64 or 128, Hq <= 32, talk not null.  The step's sequences as
 // rb_attention_prefill_bf16 takes them (cu_seqlens [B + 1], past_len [B]); steps of single tokens and of prompts alike.
+// n_splits > 1 deals every sequence's pages out to that many workgroups (for steps of few tokens with long contexts) and
+// needs a workspace of n_splits * T * Hq * (head_dim + 2) floats.
 int rb_attention_mixed_bf16(const void* q, const void* k_pages, const void* v_pages, void* out, const int32_t* cu_seqlens,
                             const int32_t* past_len, const int32_t* block_table, int bt_stride, int n_seqs, int n_tokens,
                             int n_heads, int n_kv_heads, int head_dim, float scale, const float* talk, int chunk, int window,
-                            void* stream);
+                            int n_splits, float* workspace, void* stream);
 
 // ---- attention through a latent (latent.hip)
 // Per token: cq = rmsnorm(proj[t, 0:q_rank]) * q_gain -> cq [T, q_rank]; rmsnorm(proj[t, kv_col:+kv_rank]) * kv_gain ->

@@ -182,7 +182,7 @@ class Kernels:
             "rb_scale": [_P, _F, _L, _P],
             "rb_bias_norm_store": [_P, _L, _P, _I, _F, _P, _P, _P, _I, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _P],
             "rb_attention_mixed": [_P, _P, _P, _P, _I, _P, _P, _P, _I, _I, _I, _I, _I, _F, _P, _I, _I, _P],
-            "rb_attention_mixed_bf16": [_P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _P, _I, _I, _P],
+            "rb_attention_mixed_bf16": [_P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _P, _I, _I, _I, _P, _P],
         }
         for name, args in sig.items():
             fn = getattr(L, name)
@@ -908,9 +908,10 @@ class Kernels:
                                               float(scale), _ptr(talk), int(chunk or 0), int(window or 0), self._stream()))
 
     def attention_mixed_bf16(self, q, k_pages, v_pages, out, ctx, block_table, n_heads, n_kv, head_dim, scale, talk, chunk,
-                             window) -> None:
+                             window, n_splits: int = 1, workspace: Optional[torch.Tensor] = None) -> None:
         """attention_mixed on the matrix cores: bfloat16, head_dim 64 or 128, at most 32 heads; the step's sequences from
-        ctx (cu_seqlens, past_len)."""
+        ctx (cu_seqlens, past_len).  n_splits > 1: every sequence's pages are dealt out to that many workgroups, whose sums
+        go through `workspace` (float32, n_splits * T * heads * (head_dim + 2))."""
         n = q.shape[0]
         _check(q, "q", torch.bfloat16, (n, n_heads, head_dim))
         _check(k_pages, "k_pages", torch.bfloat16)
@@ -928,10 +929,18 @@ class Kernels:
         if block_table.shape[0] < ctx.n_seqs:
             raise KernelError("attention_mixed_bf16: the block table has fewer rows than the step has sequences")
         _check(talk, "talk", torch.float32, (n_heads, n_heads))
+        n_splits = int(n_splits)
+        if not 1 <= n_splits <= 64:
+            raise KernelError(f"attention_mixed_bf16: {n_splits} splits not supported (1 to 64)")
+        if n_splits > 1:
+            _check(workspace, "workspace", torch.float32)
+            if workspace.numel() < n_splits * n * n_heads * (head_dim + 2):
+                raise KernelError("attention_mixed_bf16: the workspace is smaller than splits * T * heads * (head_dim + 2)")
         self._ok(self._lib.rb_attention_mixed_bf16(_ptr(q), _ptr(k_pages), _ptr(v_pages), _ptr(out), _ptr(ctx.cu_seqlens),
                                                    _ptr(ctx.past_len), _ptr(block_table), block_table.shape[1], ctx.n_seqs, n,
                                                    n_heads, n_kv, head_dim, float(scale), _ptr(talk), int(chunk or 0),
-                                                   int(window or 0), self._stream()))
+                                                   int(window or 0), n_splits, _ptr(workspace) if n_splits > 1 else None,
+                                                   self._stream()))
 
     def pairs_sum(self, pairs: torch.Tensor, top: int, out: torch.Tensor) -> None:
         n, width = out.shape

@@ -194,6 +194,17 @@ class StepContext:
                 self._copied = torch.cuda.Event()
             self._copied.record()
 
+    def tile_split_workspace(self, n_heads: int, head_dim: int, pages_per_split: int = 2) -> Tuple:
+        """Split count and scratch for an attention kernel whose workgroup takes ALL heads of a sequence and to which a
+        page costs much (several barriers): a step of single tokens deals the pages out, about `pages_per_split` to a
+        workgroup at the short end of a context bucket (a bucket holds 8 to 16 pages per split of ordinary decode attention)."""
+        n_splits = max(1, min(16, (8 // pages_per_split) * int(self.bucket), self.n_compute_units // max(1, self.n_seqs)))
+        key = ("tiles", n_heads, head_dim, n_splits)
+        if key not in self._workspaces:
+            ws = torch.empty(self.n_seqs * n_heads * n_splits * (head_dim + 2), dtype=torch.float32, device=self.device)
+            self._workspaces[key] = (n_splits, ws)
+        return self._workspaces[key]
+
     def decode_workspace(self, n_heads: int, head_dim: int, n_kv_heads: int = 1) -> Tuple:
         """Split count and scratch for decode attention: enough workgroups to fill the
         GPU, whatever the context length (each split strides over the pages)."""

@@ -208,8 +208,10 @@ class Attention(Part):
         attn = torch.empty((t, hq * d), dtype=self.env.dtype, device=h.device)
         window = int(self.window) if self.window is not None else 0
         if self.mixed_on_matrix_cores:
+            # a step of single tokens: every sequence's pages dealt out to several workgroups
+            n_splits, ws = ctx.tile_split_workspace(hq, d) if t == ctx.n_seqs else (1, None)
             lib.attention_mixed_bf16(q, view.k_pages, view.v_pages, attn, ctx, view.block_table, hq, hk, d, self.scale, self.talk,
-                                     self.chunk or 0, window)
+                                     self.chunk or 0, window, n_splits, ws)
         else:
             lib.attention_mixed(q, view.k_pages, view.v_pages, attn, ctx.tok_pos, ctx.tok_seq, view.block_table, hq, hk, d,
                                 self.scale, self.talk, self.chunk or 0, window)
