@@ -116,12 +116,15 @@ __global__ __launch_bounds__(64 * NW) void attention_mixed_mfma_kernel(
   const int hpw = (n_heads + NW - 1) / NW;
   const int h_lo = wave * hpw, h_hi = h_lo + hpw < n_heads ? h_lo + hpw : n_heads;
   const size_t q_row = ((size_t)(seq_start + q0 + (l16 < n_valid ? l16 : n_valid - 1)) * n_heads) * D + lg * 8;
-  Frag8 qres[HW * (D / 32)];
+  constexpr bool QRES = HW * (D / 32) <= 8;        // the wave's queries stay in registers for all tiles
+  Frag8 qres[QRES ? HW * (D / 32) : 1];
+  if (QRES) {
 #pragma unroll
-  for (int k = 0; k < HW; ++k)
+    for (int k = 0; k < HW; ++k)
 #pragma unroll
-    for (int s = 0; s < D / 32; ++s)
-      qres[k * (D / 32) + s].u = h_lo + k < h_hi ? load16(q + q_row + (size_t)(h_lo + k) * D + s * 32) : zero16();
+      for (int s = 0; s < D / 32; ++s)
+        qres[k * (D / 32) + s].u = h_lo + k < h_hi ? load16(q + q_row + (size_t)(h_lo + k) * D + s * 32) : zero16();
+  }
 
   // ---- V^T of a tile and gv kv heads: a thread takes 4 keys in a row and 8 numbers of each, and writes 8 times 4 keys
   constexpr int VU = 16 * (D / 8);                  // threads a kv head
@@ -153,17 +156,18 @@ __global__ __launch_bounds__(64 * NW) void attention_mixed_mfma_kernel(
   // ---- the 64 keys of a tile and kv head as B operands, asked for together; where registers allow (heads of 64), those
   // of the wave's first kv head are asked for a tile ahead
   constexpr bool KP = D == 64;
-  Frag8 kf[4][D / 32];
+  constexpr int KBL = KP ? 4 : 1;                  // key blocks of 16 asked for together
+  Frag8 kf[KBL][D / 32];
   int g_have = -1;
-  auto load_k = [&](int kt, int g) {
-    const bf16_t* krow = k_pages + (((size_t)bt[kt] * n_kv + g) * RB_PAGE + l16) * D + lg * 8;
+  auto load_k = [&](int kt, int g, int kb0) {
+    const bf16_t* krow = k_pages + (((size_t)bt[kt] * n_kv + g) * RB_PAGE + kb0 * 16 + l16) * D + lg * 8;
 #pragma unroll
-    for (int kb = 0; kb < 4; ++kb)
+    for (int kb = 0; kb < KBL; ++kb)
 #pragma unroll
       for (int s = 0; s < D / 32; ++s) kf[kb][s].u = load16(krow + (size_t)kb * 16 * D + s * 32);
     g_have = g;
   };
-  if (KP && first_tile <= last_tile && h_lo < h_hi) load_k(first_tile, h_lo / group);
+  if (KP && first_tile <= last_tile && h_lo < h_hi) load_k(first_tile, h_lo / group, 0);
   if (first_tile <= last_tile) load_v(first_tile, 0);
 
   for (int kt = first_tile; kt <= last_tile; kt += n_splits) {
@@ -179,14 +183,22 @@ __global__ __launch_bounds__(64 * NW) void attention_mixed_mfma_kernel(
         const int h = h_lo + k;
         if (h < h_hi) {
           const int g = h / group;
-          if (g != g_have) load_k(kt, g);
-          const Frag8* qf = qres + k * (D / 32);
+          if (KP && g != g_have) load_k(kt, g, 0);
+          Frag8 qf[D / 32];
+#pragma unroll
+          for (int s = 0; s < D / 32; ++s) {
+            if (QRES)
+              qf[s] = qres[k * (D / 32) + s];
+            else
+              qf[s].u = load16(q + q_row + (size_t)h * D + s * 32);
+          }
           float* dst = S + (size_t)h * TM_HEAD + l16;
 #pragma unroll
           for (int kb = 0; kb < 4; ++kb) {
+            if (!KP) load_k(kt, g, kb);
             f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-            for (int s = 0; s < D / 32; ++s) acc = mfma16(qf[s], kf[kb][s], acc);
+            for (int s = 0; s < D / 32; ++s) acc = mfma16(qf[s], kf[KP ? kb : 0][s], acc);
             if (full) {
 #pragma unroll
               for (int r = 0; r < 4; ++r) dst[(4 * lg + r) * TM_ROW + kb * 16] = acc[r] * scale_log2;
@@ -202,7 +214,7 @@ __global__ __launch_bounds__(64 * NW) void attention_mixed_mfma_kernel(
           }
         }
       }
-      if (KP && kt + n_splits <= last_tile && h_lo < h_hi) load_k(kt + n_splits, h_lo / group);
+      if (KP && kt + n_splits <= last_tile && h_lo < h_hi) load_k(kt + n_splits, h_lo / group, 0);
     }
     __syncthreads();
     // ---------------------------------------------------------------- 2. mixing over the heads

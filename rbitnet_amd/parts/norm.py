@@ -48,10 +48,6 @@ class RMSNorm(Part):
     def tensor_specs(self) -> Dict[str, TensorSpec]:
         return {self.names["weight"]: TensorSpec(() if self.scalar else (self.size,), role="gain", init="ones_normal")}
 
-    def tensor_names(self, base: str) -> Dict[str, str]:
-        """full name -> the part's own name, for an owner that stores the norm under `base`."""
-        return {".".join(p for p in (base, name) if p): name for name in self.tensor_specs()}
-
     def load(self, tensors: Dict[str, torch.Tensor]) -> None:
         w = tensors[self.names["weight"]]
         self.weight = w.reshape(1).expand(self.size).contiguous() if self.scalar else w
