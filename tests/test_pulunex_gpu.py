@@ -573,7 +573,7 @@ def test_long_decoding_and_greedy_generation_through_the_engine(name, dtype):
         same = sum(1 for g, t, c in zip(greedy, r.tokens, clear.tolist()) if c and g == t)
         assert same >= (1.0 if dtype == "float32" else 0.9) * int(clear.sum())
         assert int(clear.sum()) > (0.9 if dtype == "float32" else 0.4) * n
-    assert eng.stats["decode_tokens"] > 0
+    assert eng.stats["decode_tokens"] > 0 and eng.model.graph_safe and eng.model.plan_safe
 
 
 def test_replay_and_command_line_on_a_model_of_this_design(tmp_path, capsys):
