@@ -194,7 +194,7 @@ class StepContext:
                 self._copied = torch.cuda.Event()
             self._copied.record()
 
-    def tile_split_workspace(self, n_heads: int, head_dim: int, pages_per_split: int = 2) -> Tuple:
+    def tile_split_workspace(self, n_heads: int, head_dim: int, pages_per_split: int = 1) -> Tuple:
         """Split count and scratch for an attention kernel whose workgroup takes ALL heads of a sequence and to which a
         page costs much (several barriers): a step of single tokens deals the pages out, about `pages_per_split` to a
         workgroup at the short end of a context bucket (a bucket holds 8 to 16 pages per split of ordinary decode attention)."""

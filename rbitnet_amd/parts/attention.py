@@ -208,8 +208,14 @@ class Attention(Part):
         attn = torch.empty((t, hq * d), dtype=self.env.dtype, device=h.device)
         window = int(self.window) if self.window is not None else 0
         if self.mixed_on_matrix_cores:
-            # a step of single tokens: every sequence's pages dealt out to several workgroups
-            n_splits, ws = ctx.tile_split_workspace(hq, d) if t == ctx.n_seqs else (1, None)
+            # a step of single tokens: every sequence's pages dealt out to several workgroups; so are those of a prompt
+            # whose 16-query tiles leave compute units idle (the last tiles of a prompt walk the most pages)
+            if t == ctx.n_seqs:
+                n_splits, ws = ctx.tile_split_workspace(hq, d)
+            else:
+                tiles = t // 16 + ctx.n_seqs
+                n_splits = max(1, min(4, (lib.n_compute_units + tiles // 2) // tiles))
+                ws = torch.empty(n_splits * t * hq * (d + 2), dtype=torch.float32, device=h.device) if n_splits > 1 else None
             lib.attention_mixed_bf16(q, view.k_pages, view.v_pages, attn, ctx, view.block_table, hq, hk, d, self.scale, self.talk,
                                      self.chunk or 0, window, n_splits, ws)
         else:
