@@ -116,7 +116,7 @@ __global__ __launch_bounds__(64 * NW) void attention_mixed_mfma_kernel(
   const int hpw = (n_heads + NW - 1) / NW;
   const int h_lo = wave * hpw, h_hi = h_lo + hpw < n_heads ? h_lo + hpw : n_heads;
   const size_t q_row = ((size_t)(seq_start + q0 + (l16 < n_valid ? l16 : n_valid - 1)) * n_heads) * D + lg * 8;
-  constexpr bool QRES = HW * (D / 32) <= 8;        // the wave's queries stay in registers for all tiles
+  constexpr bool QRES = HW * (D / 32) <= 4;        // the wave's queries stay in registers for all tiles
   Frag8 qres[QRES ? HW * (D / 32) : 1];
   if (QRES) {
 #pragma unroll
