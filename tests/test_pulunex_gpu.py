@@ -339,6 +339,34 @@ def test_a_far_key_among_hundreds(lib, dtype):
             assert _close(got[600:], want[600:], dtype), (mask, cuts)
 
 
+@pytest.mark.parametrize("heads,kv_heads,dim,chunk", [(6, 3, 64, 100), (16, 4, 64, 0), (32, 8, 64, 70), (8, 1, 128, 0), (20, 4, 128, 200)])
+def test_matrix_core_kernel_for_any_number_of_splits_against_the_kernel_for_any_sizes(lib, heads, kv_heads, dim, chunk):
+    """The two kernels on the same bfloat16 queries and pages: three sequences that go on at unequal lengths with unequal
+    numbers of new tokens (a page's border, one token, more than 16), the pages dealt out to 1, 2, 3 and 16 workgroups."""
+    from rbitnet_amd.parts import CacheRequest
+    cache = Cache([CacheRequest("kv", heads=kv_heads, head_dim=dim)], 3, 64 * 24, torch.bfloat16, DEV)
+    slots = [cache.alloc_slot() for _ in range(3)]
+    past, new = [130, 0, 447], [40, 1, 17]
+    cache.reserve(slots, past)
+    cache.commit(slots, past)
+    ctx = _step(lib, cache, slots, new)
+    view = cache.view(0, ctx.block_tables)
+    view.k_pages.normal_()
+    view.v_pages.normal_()
+    n = sum(new)
+    q = torch.randn(n, heads, dim, device=DEV).to(torch.bfloat16)
+    talk = (torch.eye(heads, device=DEV) + 0.3 * torch.randn(heads, heads, device=DEV)).contiguous()
+    want = torch.empty(n, heads * dim, dtype=torch.float32, device=DEV)
+    lib.attention_mixed(q.float(), view.k_pages.float(), view.v_pages.float(), want, ctx.tok_pos, ctx.tok_seq, view.block_table, heads,
+                        kv_heads, dim, 0.11, talk, chunk, 0)
+    for n_splits in (1, 2, 3, 16):
+        got = torch.full((n, heads * dim), float("nan"), dtype=torch.bfloat16, device=DEV)
+        ws = torch.empty(n_splits * n * heads * (dim + 2), dtype=torch.float32, device=DEV) if n_splits > 1 else None
+        lib.attention_mixed_bf16(q, view.k_pages, view.v_pages, got, ctx, view.block_table, heads, kv_heads, dim, 0.11, talk, chunk, 0,
+                                 n_splits, ws)
+        assert _rel(got, want) < 6e-3, n_splits            # the output's rounding to bfloat16
+
+
 # ---------------------------------------------------------------------------- feed-forwards
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("hidden,ff", [(64, 172), (48, 20), (128, 256)])
