@@ -579,6 +579,7 @@ def test_batches_of_unequal_requests_and_slots_used_again(name, dtype):
             g = torch.cat(got[i])
             assert _close_rows(g, want[i][:g.shape[0]], dtype), (wave, i)
         eng.cache.check()
+    assert eng.plans.stats["replayed"] > 0          # steps of a shape that came back were issued from their recording
 
 
 @pytest.mark.parametrize("name,dtype", [("A", "float32"), ("C", "bfloat16")])
