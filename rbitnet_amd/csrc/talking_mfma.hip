@@ -63,7 +63,7 @@ __global__ __launch_bounds__(64 * NW) void attention_mixed_mfma_kernel(
     q_len = cu_seqlens[b + 1] - seq_start;
     const int tiles = (q_len + TM_Q - 1) / TM_Q;
     if (wg < tiles) {
-      q0 = wg * TM_Q;
+      q0 = (tiles - 1 - wg) * TM_Q;        // a sequence's last queries walk the most pages: they start first
       break;
     }
     wg -= tiles;
