@@ -68,7 +68,7 @@ class PagedGroup:
         self.request = request
         self.layers = list(layers)
         self.index = {l: i for i, l in enumerate(self.layers)}
-        self.table = PageTable(n_pages, request.window)
+        self.table = PageTable(n_pages, request.window, getattr(request, "keep_first", 0))
         self.spare_page = int(n_pages)
 
     def open(self, slot: int) -> None:

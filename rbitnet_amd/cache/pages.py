@@ -74,11 +74,13 @@ class PageTable:
     """The pages of each slot for one storage group.  Logical page i of a slot covers
     positions [i * PAGE_SIZE, (i + 1) * PAGE_SIZE).  With a window, pages that lie wholly
     behind every future query's reach are given back early; their entries stay in the
-    table as -1 and are never read."""
+    table as -1 and are never read.  `keep_first` tokens at a sequence's start stay in reach
+    whatever the window: the pages that hold them are never given back early."""
 
-    def __init__(self, n_pages: int, window: Optional[int] = None):
+    def __init__(self, n_pages: int, window: Optional[int] = None, keep_first: int = 0):
         self.pool = FreeList(n_pages, "cache page")
         self.window = window
+        self.keep_first = max(0, int(keep_first or 0))
         self.tables: Dict[int, List[int]] = {}
 
     def open(self, slot: int) -> None:
@@ -109,7 +111,7 @@ class PageTable:
         dead_pages = max(0, length - self.window + 1) // PAGE_SIZE
         table = self.tables[slot]
         n = 0
-        for i in range(min(dead_pages, len(table))):
+        for i in range(pages_for(self.keep_first), min(dead_pages, len(table))):
             if table[i] >= 0:
                 self.pool.give_back(table[i])
                 table[i] = -1

@@ -19,6 +19,7 @@ from typing import Any, Dict, Iterable, Optional, Tuple
 from ..errors import ConfigError
 from .bagonex import BagonexConfig
 from .llama import LlamaConfig
+from .menerax import MeneraxConfig
 from .pulunex import PulunexConfig
 from .tigutar import TigutarConfig
 from .spec import ModelSpec
@@ -99,3 +100,4 @@ register_architecture("LlamaForCausalLM", LlamaConfig)
 register_architecture("Bagonex", BagonexConfig)
 register_architecture("Tigutar", TigutarConfig)
 register_architecture("Pulunex", PulunexConfig)
+register_architecture("Menerax", MeneraxConfig)

@@ -299,6 +299,74 @@ int rb_latent_norm_store(const float* proj, long long stride, int q_rank, const 
 int rb_heads_linear(const void* x, int x_dtype, const void* w, int w_dtype, void* y, int y_dtype, int n_tokens, int n_heads,
                     int n, int k, void* stream);
 
+// ---- a norm on the sublayer's output, limits in the gated unit, and what the mixers of such layers need
+// x <- (assign ? 0 : x) + y / sqrt(mean(y^2) + eps) * gain with y = sa * a + sb * b (b null: sa * a), rows of `width` float32
+// numbers; h_out (null: none) gets the new rows of x in h_dtype.
+int rb_outnorm_residual(float* x, const float* a, const float* b, float sa, float sb, const float* gain, float eps, int assign,
+                        void* h_out, int h_dtype, int n_tokens, int width, void* stream);
+// g = min(gu[r, j], limit), u = clamp(gu[r, F + j], -limit, limit); out[r, j] = g sigmoid(alpha g) (u + 1).  limit <= 0: none.
+int rb_clamped_glu(const float* gu, void* out, int out_dtype, int n_rows, int ff, float limit, float alpha, void* stream);
+// out = tanh(z), n numbers.
+int rb_tanh_cast(const float* z, void* out, int out_dtype, long long n, void* stream);
+// rb_attention_generic_sinks with kept first keys behind the window (j < keep_first stays visible) and capped scores
+// (softcap > 0: s <- softcap tanh(s / softcap) after the scale).
+int rb_attention_generic_opts(const void* q, const void* k_pages, const void* v_pages, void* out, int dtype,
+                              const int32_t* tok_pos, const int32_t* tok_seq, const int32_t* block_table, int bt_stride,
+                              int n_tokens, int n_heads, int n_kv_heads, int head_dim, float scale, int window, int keep_first,
+                              float softcap, const float* sinks, void* stream);
+// The matrix-core kernels with the same two choices (see rb_attention_prefill_bf16_sinks, rb_attention_decode_bf16_sinks).
+int rb_attention_prefill_bf16_opts(const void* q, const void* k_pages, const void* v_pages, void* out,
+                                   const int32_t* cu_seqlens, const int32_t* past_len, const int32_t* block_table,
+                                   int bt_stride, int n_seqs, int max_q_len, int n_heads, int n_kv_heads, int head_dim,
+                                   float scale, int window, int keep_first, float softcap, const float* sinks, void* stream);
+int rb_attention_decode_bf16_opts(const void* q, const void* k_pages, const void* v_pages, void* out,
+                                  const int32_t* tok_pos, const int32_t* block_table, int bt_stride, int n_seqs,
+                                  int n_heads, int n_kv_heads, int head_dim, float scale, int window, int keep_first,
+                                  float softcap, int n_splits, float* workspace, const float* sinks, void* stream);
+// rb_rope_store with every query and key head RMS-normed first over its dim numbers, x / sqrt(mean(x^2) + eps) * w, with a
+// weight of dim numbers that the heads share (q_norm, k_norm float32 [dim]).
+int rb_norm_rope_store(const float* qkv, long long row_width, const float* cos, const float* sin, int rot, const float* q_norm,
+                       const float* k_norm, float eps, void* q_out, void* k_pages, void* v_pages, int cache_dtype,
+                       const int32_t* tok_pos, const int32_t* tok_seq, const int32_t* block_table, int bt_stride, int n_tokens,
+                       int n_heads, int n_kv_heads, int dim, int vdim, int pad, void* stream);
+// x[e] *= sigmoid(gate[e]) for n numbers, x of dtype, gate float32, laid out alike.
+int rb_sigmoid_gate(void* x, int dtype, const float* gate, long long n, void* stream);
+// out[m, t, :] = h[t] + (h[t - 1] - h[t]) * mu[m] for m < n_mix (mu float32 [n_mix, E]); the row before a step's first
+// comes from state [slots, E] (float32), which then holds the step's last row.  h and out [n_mix, T, E] of dtype.
+int rb_shift_mix(const void* h, int dtype, float* state, const float* mu, int n_mix, void* out, const int32_t* cu_seqlens,
+                 const int32_t* tok_seq, const int32_t* slots, int n_tokens, int n_seqs, int width, void* stream);
+// rb_short_conv on x + bias (float32 [C], null: none); the state holds the inputs with their bias.
+int rb_short_conv_bias(const float* x, long long x_stride, const float* bias, const float* w, int taps, float* state,
+                       const int32_t* tok_pos, const int32_t* tok_seq, const int32_t* cu_seqlens, const int32_t* slots, void* out,
+                       long long out_stride, int out_dtype, int residual, int act, int n_tokens, int n_seqs, int channels,
+                       void* stream);
+// rb_recurrence_prep takes decay 2 as well: exp(-exp(a + bias[i])).
+// rb_linear_recurrence read before the token's write, with a weight per head and key channel on the token's own k v^T
+// (bonus float32 [H, dim]; null: rb_linear_recurrence):  out = (S + diag(bonus) k v^T)^T q;  S <- diag(g) S + k v^T.
+int rb_linear_recurrence_bonus(const float* q, const float* k, long long qk_stride, const float* v, long long v_stride,
+                               const float* g, long long g_stride, int g_per_head, const float* beta, const float* bonus,
+                               float* state, const int32_t* cu_seqlens, const int32_t* slots, float* out, int n_seqs, int n_tokens,
+                               int n_heads, int n_kv_heads, int dim, int vdim, void* stream);
+// rb_gated_rmsnorm_act with head h's weight at weight + h * weight_head_stride (0: one weight for all heads).
+int rb_gated_rmsnorm_heads(const float* o, const float* weight, long long weight_head_stride, const float* gate,
+                           long long gate_stride, int act, float eps, void* out, int out_dtype, int n_tokens, int n_heads, int vdim,
+                           void* stream);
+// rb_heads_linear on a part of every head: a head of x takes x_head_stride numbers (the first k are read), a head of y
+// y_head_stride (the first n are written).
+int rb_heads_linear_strided(const void* x, int x_dtype, long long x_head_stride, const void* w, int w_dtype, void* y, int y_dtype,
+                            long long y_head_stride, int n_tokens, int n_heads, int n, int k, void* stream);
+// rb_latent_norm_store into pages [n_pages, 1, 64, page_width] with, behind the latent, the `rot` numbers at rot_col of the
+// row rotated by the token's position (style 0: 2i with 2i + 1; 1: i with i + rot / 2) and zeros up to page_width.
+int rb_latent_norm_rope_store(const float* proj, long long stride, int q_rank, const float* q_gain, void* cq, int kv_col,
+                              int kv_rank, const float* kv_gain, void* pages, int page_width, int rot_col, int rot, const float* cos,
+                              const float* sin, int style, int dtype, const int32_t* tok_pos, const int32_t* tok_seq,
+                              const int32_t* block_table, int bt_stride, float eps, int n_tokens, void* stream);
+// Of every head of x [T, H, x_head_stride] float32 the `rot` numbers at x_col, rotated by the token's position, go to
+// y [T, H, y_head_stride] at y_col; what lies behind them in a head of y becomes zero.
+int rb_rope_heads_part(const float* x, long long x_head_stride, int x_col, int rot, const float* cos, const float* sin, int style,
+                       void* y, int y_dtype, long long y_head_stride, int y_col, const int32_t* tok_pos, int n_tokens, int n_heads,
+                       void* stream);
+
 // tokens[r] = argmax of logits[r, :] (NaN counts as -inf, lowest index among equals), or, where
 // temperature[r] > 0, the first index whose running sum of exp(z/T - max) reaches u[r] times the total.
 // workspace: rb_sample_workspace_bytes(n_rows, vocab) bytes, 8-byte aligned, contents do not matter.

@@ -25,7 +25,7 @@ __global__ __launch_bounds__(RB_WAVE * AG_MAX_WAVES) void attention_generic_kern
     const T* __restrict__ q, const T* __restrict__ k_pages, const T* __restrict__ v_pages, T* __restrict__ out,
     const int32_t* __restrict__ tok_pos, const int32_t* __restrict__ tok_seq,
     const int32_t* __restrict__ block_table, int bt_stride, int n_heads, int n_kv, int head_dim, float scale,
-    int window, const float* __restrict__ sinks) {
+    int window, const float* __restrict__ sinks, int keep_first, float softcap) {
   __shared__ float qs[AG_MAX_D];
   __shared__ float ps_all[AG_MAX_WAVES][RB_PAGE];
   __shared__ float red_m[AG_MAX_WAVES], red_l[AG_MAX_WAVES];
@@ -49,15 +49,23 @@ __global__ __launch_bounds__(RB_WAVE * AG_MAX_WAVES) void attention_generic_kern
 #pragma unroll
   for (int i = 0; i < AG_MAX_D / RB_WAVE; ++i) acc[i] = 0.f;
 
-  for (int pg = lo / RB_PAGE + wave; pg <= pos / RB_PAGE; pg += n_waves) {
+  // the pages that hold visible keys: those of the kept first tokens that lie before the window's first page, then the
+  // window's (every one of them holds at least one visible key)
+  const int lo_page = lo / RB_PAGE;
+  const int kept_pages = keep_first > 0 ? (keep_first + RB_PAGE - 1) / RB_PAGE : 0;
+  const int n_first = kept_pages < lo_page ? kept_pages : lo_page;
+  const int n_walk = n_first + pos / RB_PAGE - lo_page + 1;
+  for (int walk = wave; walk < n_walk; walk += n_waves) {
+    const int pg = walk < n_first ? walk : lo_page + walk - n_first;
     const size_t base = ((size_t)pages[pg] * n_kv + kvh) * RB_PAGE * head_dim;
     const int p = pg * RB_PAGE + lane;
     float s = -INFINITY;
-    if (p >= lo && p <= pos) {
+    if (p <= pos && (p >= lo || p < keep_first)) {
       const T* krow = k_pages + base + (size_t)lane * head_dim;
       float dot = 0.f;
       for (int d = 0; d < head_dim; ++d) dot = fmaf(qs[d], Num<T>::load(krow + d), dot);
       s = dot * scale;
+      if (softcap > 0.f) s = softcap * tanhf(s / softcap);
     }
     const float m_new = fmaxf(m_run, wave_max(s));      // finite: the page holds at least one valid key
     const float pexp = (s == -INFINITY) ? 0.f : expf(s - m_new);
@@ -67,7 +75,7 @@ __global__ __launch_bounds__(RB_WAVE * AG_MAX_WAVES) void attention_generic_kern
     // ps belongs to this wave alone; a wave's LDS accesses complete in order
     ps[lane] = pexp;
     __builtin_amdgcn_wave_barrier();
-    const int j_lo = (pg * RB_PAGE < lo) ? lo - pg * RB_PAGE : 0;
+    const int j_lo = (pg * RB_PAGE < lo && pg * RB_PAGE >= keep_first) ? lo - pg * RB_PAGE : 0;      // keys between carry weight 0
     const int j_hi = (pg * RB_PAGE + RB_PAGE - 1 > pos) ? pos - pg * RB_PAGE : RB_PAGE - 1;
 #pragma unroll
     for (int i = 0; i < AG_MAX_D / RB_WAVE; ++i) {
@@ -146,7 +154,7 @@ __global__ __launch_bounds__(RB_WAVE * AG_MAX_WAVES) void attention_generic_vec_
     const T* __restrict__ q, const T* __restrict__ k_pages, const T* __restrict__ v_pages, T* __restrict__ out,
     const int32_t* __restrict__ tok_pos, const int32_t* __restrict__ tok_seq,
     const int32_t* __restrict__ block_table, int bt_stride, int n_heads, int n_kv, int head_dim, float scale,
-    int window, int group_lanes, const float* __restrict__ sinks) {
+    int window, int group_lanes, const float* __restrict__ sinks, int keep_first, float softcap) {
   __shared__ __attribute__((aligned(16))) float qs[AG_MAX_D];
   __shared__ float ps_all[AG_MAX_WAVES][RB_PAGE];
   __shared__ float red_m[AG_MAX_WAVES], red_l[AG_MAX_WAVES];
@@ -170,11 +178,18 @@ __global__ __launch_bounds__(RB_WAVE * AG_MAX_WAVES) void attention_generic_vec_
 
   float m_run = -INFINITY, l_run = 0.f;
   float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
-  for (int pg = lo / RB_PAGE + wave; pg <= pos / RB_PAGE; pg += n_waves) {
+  // the pages that hold visible keys: those of the kept first tokens that lie before the window's first page, then the
+  // window's (every one of them holds at least one visible key)
+  const int lo_page = lo / RB_PAGE;
+  const int kept_pages = keep_first > 0 ? (keep_first + RB_PAGE - 1) / RB_PAGE : 0;
+  const int n_first = kept_pages < lo_page ? kept_pages : lo_page;
+  const int n_walk = n_first + pos / RB_PAGE - lo_page + 1;
+  for (int walk = wave; walk < n_walk; walk += n_waves) {
+    const int pg = walk < n_first ? walk : lo_page + walk - n_first;
     const size_t base = ((size_t)pages[pg] * n_kv + kvh) * RB_PAGE * head_dim;
     const int p = pg * RB_PAGE + lane;
     float s = -INFINITY;
-    if (p >= lo && p <= pos) {
+    if (p <= pos && (p >= lo || p < keep_first)) {
       const T* krow = k_pages + base + (size_t)lane * head_dim;
       float d0 = 0.f, d1 = 0.f, d2 = 0.f, d3 = 0.f;
       for (int cc = 0; cc < chunks; ++cc) {
@@ -186,6 +201,7 @@ __global__ __launch_bounds__(RB_WAVE * AG_MAX_WAVES) void attention_generic_vec_
         d3 = fmaf(qv.w, kv.w, d3);
       }
       s = ((d0 + d1) + (d2 + d3)) * scale;
+      if (softcap > 0.f) s = softcap * tanhf(s / softcap);
     }
     const float m_new = fmaxf(m_run, wave_max(s));      // finite: the page holds at least one valid key
     const float pexp = (s == -INFINITY) ? 0.f : expf(s - m_new);
@@ -194,7 +210,7 @@ __global__ __launch_bounds__(RB_WAVE * AG_MAX_WAVES) void attention_generic_vec_
     m_run = m_new;
     ps[lane] = pexp;                                    // this wave's alone; a wave's LDS accesses complete in order
     __builtin_amdgcn_wave_barrier();
-    const int j_lo = (pg * RB_PAGE < lo) ? lo - pg * RB_PAGE : 0;
+    const int j_lo = (pg * RB_PAGE < lo && pg * RB_PAGE >= keep_first) ? lo - pg * RB_PAGE : 0;      // keys between carry weight 0
     const int j_hi = (pg * RB_PAGE + RB_PAGE - 1 > pos) ? pos - pg * RB_PAGE : RB_PAGE - 1;
     acc.x *= corr;
     acc.y *= corr;
@@ -276,6 +292,21 @@ extern "C" int rb_attention_generic_sinks(const void* q, const void* k_pages, co
                                           float scale, int window, const float* sinks, void* stream) {
   RB_RECORDED(rb_attention_generic_sinks(q, k_pages, v_pages, out, dtype, tok_pos, tok_seq, block_table, bt_stride, n_tokens,
                                          n_heads, n_kv_heads, head_dim, scale, window, sinks, stream));
+  return rb_attention_generic_opts(q, k_pages, v_pages, out, dtype, tok_pos, tok_seq, block_table, bt_stride, n_tokens, n_heads,
+                                   n_kv_heads, head_dim, scale, window, 0, 0.0f, sinks, stream);
+}
+
+// The same with two more choices.  keep_first (with a window): the first keep_first keys of a sequence stay visible behind
+// the window, a query at position i seeing j <= i with i - j < window or j < keep_first.  softcap > 0: a score s becomes
+// softcap * tanh(s / softcap) after the scale and before the softmax.
+extern "C" int rb_attention_generic_opts(const void* q, const void* k_pages, const void* v_pages, void* out, int dtype,
+                                         const int32_t* tok_pos, const int32_t* tok_seq, const int32_t* block_table,
+                                         int bt_stride, int n_tokens, int n_heads, int n_kv_heads, int head_dim,
+                                         float scale, int window, int keep_first, float softcap, const float* sinks,
+                                         void* stream) {
+  RB_RECORDED(rb_attention_generic_opts(q, k_pages, v_pages, out, dtype, tok_pos, tok_seq, block_table, bt_stride, n_tokens,
+                                        n_heads, n_kv_heads, head_dim, scale, window, keep_first, softcap, sinks, stream));
+  RB_REQUIRE(keep_first >= 0 && softcap >= 0.f, "rb_attention_generic: negative keep_first or softcap");
   RB_REQUIRE(n_tokens >= 0 && n_heads > 0 && n_kv_heads > 0 && n_heads % n_kv_heads == 0,
              "rb_attention_generic: bad head counts Hq=%d Hk=%d", n_heads, n_kv_heads);
   RB_REQUIRE(head_dim > 0 && head_dim <= AG_MAX_D, "rb_attention_generic: head_dim %d not supported (at most %d)", head_dim,
@@ -297,12 +328,12 @@ extern "C" int rb_attention_generic_sinks(const void* q, const void* k_pages, co
       attention_generic_vec_kernel<float><<<grid, threads, 0, s>>>((const float*)q, (const float*)k_pages,
                                                                   (const float*)v_pages, (float*)out, tok_pos, tok_seq,
                                                                   block_table, bt_stride, n_heads, n_kv_heads, head_dim,
-                                                                  scale, window, group_lanes, sinks);
+                                                                  scale, window, group_lanes, sinks, keep_first, softcap);
     else
       attention_generic_vec_kernel<bf16_t><<<grid, threads, 0, s>>>((const bf16_t*)q, (const bf16_t*)k_pages,
                                                                    (const bf16_t*)v_pages, (bf16_t*)out, tok_pos,
                                                                    tok_seq, block_table, bt_stride, n_heads, n_kv_heads,
-                                                                   head_dim, scale, window, group_lanes, sinks);
+                                                                   head_dim, scale, window, group_lanes, sinks, keep_first, softcap);
     RB_LAUNCH_CHECK();
     return 0;
   }
@@ -310,12 +341,12 @@ extern "C" int rb_attention_generic_sinks(const void* q, const void* k_pages, co
     attention_generic_kernel<float><<<grid, threads, 0, s>>>((const float*)q, (const float*)k_pages,
                                                             (const float*)v_pages, (float*)out, tok_pos, tok_seq,
                                                             block_table, bt_stride, n_heads, n_kv_heads, head_dim,
-                                                            scale, window, sinks);
+                                                            scale, window, sinks, keep_first, softcap);
   else if (dtype == RB_BF16)
     attention_generic_kernel<bf16_t><<<grid, threads, 0, s>>>((const bf16_t*)q, (const bf16_t*)k_pages,
                                                              (const bf16_t*)v_pages, (bf16_t*)out, tok_pos,
                                                              tok_seq, block_table, bt_stride, n_heads, n_kv_heads,
-                                                             head_dim, scale, window, sinks);
+                                                             head_dim, scale, window, sinks, keep_first, softcap);
   else
     RB_REQUIRE(false, "rb_attention_generic: unknown dtype %d", dtype);
   RB_LAUNCH_CHECK();

@@ -449,3 +449,167 @@ extern "C" int rb_swiglu(const float* gu, void* out, int out_dtype, int n_rows, 
   RB_LAUNCH_CHECK();
   return 0;
 }
+
+// ---------------------------------------------------------------- a norm on a sublayer's output, with the residual sum
+// A layer whose norm stands on the sublayer's output: x <- x + y / sqrt(mean(y^2) + eps) * gain with y = sa * a + sb * b
+// (b null: y = sa * a), all in float32; `assign` writes the normed y over x instead of adding it (the norm behind an
+// embedding).  h_out (null: none) gets the new row of x in the compute dtype, which is what the next sublayer reads.
+// One workgroup a row; a row of up to 4 * THREADS numbers stays in registers between the two passes.
+template <typename TO>
+__global__ __launch_bounds__(1024) void outnorm_residual_kernel(float* __restrict__ x, const float* __restrict__ a,
+                                                                const float* __restrict__ b, float sa, float sb,
+                                                                const float* __restrict__ gain, float eps, int assign,
+                                                                TO* __restrict__ h_out, int width) {
+  __shared__ float scratch[16];
+  const size_t r = blockIdx.x;
+  const float* ar = a + r * width;
+  const float* br = b ? b + r * width : nullptr;
+  float ss = 0.f;
+  for (int j = threadIdx.x; j < width; j += blockDim.x) {
+    float y = sa * ar[j];
+    if (br) y = fmaf(sb, br[j], y);
+    ss = fmaf(y, y, ss);
+  }
+  const float f = 1.0f / sqrtf(block_sum(ss, scratch) / (float)width + eps);
+  for (int j = threadIdx.x; j < width; j += blockDim.x) {
+    float y = sa * ar[j];
+    if (br) y = fmaf(sb, br[j], y);
+    const float n = y * f * gain[j];
+    const float v = assign ? n : x[r * width + j] + n;
+    x[r * width + j] = v;
+    if (h_out) Num<TO>::store(h_out + r * width + j, v);
+  }
+}
+
+template <typename TO>
+__global__ __launch_bounds__(1024) void outnorm_residual_vec_kernel(float* __restrict__ x, const float* __restrict__ a,
+                                                                    const float* __restrict__ b, float sa, float sb,
+                                                                    const float* __restrict__ gain, float eps, int assign,
+                                                                    TO* __restrict__ h_out, int width) {
+  __shared__ float scratch[16];
+  const size_t r = blockIdx.x;
+  const float* ar = a + r * width;
+  const float* br = b ? b + r * width : nullptr;
+  const int j0 = 4 * threadIdx.x;
+  auto term = [&](int j) {
+    float4 y = *reinterpret_cast<const float4*>(ar + j);
+    y = make_float4(sa * y.x, sa * y.y, sa * y.z, sa * y.w);
+    if (br) {
+      const float4 z = *reinterpret_cast<const float4*>(br + j);
+      y = make_float4(fmaf(sb, z.x, y.x), fmaf(sb, z.y, y.y), fmaf(sb, z.z, y.z), fmaf(sb, z.w, y.w));
+    }
+    return y;
+  };
+  float4 keep = make_float4(0.f, 0.f, 0.f, 0.f);
+  float ss = 0.f;
+  for (int j = j0; j < width; j += 4 * blockDim.x) {
+    const float4 y = term(j);
+    if (j == j0) keep = y;
+    ss += (y.x * y.x + y.y * y.y) + (y.z * y.z + y.w * y.w);
+  }
+  const float f = 1.0f / sqrtf(block_sum(ss, scratch) / (float)width + eps);
+  for (int j = j0; j < width; j += 4 * blockDim.x) {
+    const float4 y = j == j0 ? keep : term(j);
+    const float4 g = *reinterpret_cast<const float4*>(gain + j);
+    float4 v = make_float4(y.x * f * g.x, y.y * f * g.y, y.z * f * g.z, y.w * f * g.w);
+    if (!assign) {
+      const float4 o = *reinterpret_cast<const float4*>(x + r * width + j);
+      v = make_float4(o.x + v.x, o.y + v.y, o.z + v.z, o.w + v.w);
+    }
+    *reinterpret_cast<float4*>(x + r * width + j) = v;
+    if (h_out) {
+      if (sizeof(TO) == 4)
+        *reinterpret_cast<float4*>(h_out + r * width + j) = v;
+      else
+        *reinterpret_cast<uint2*>(h_out + r * width + j) = make_uint2(pack_bf16x2(v.x, v.y), pack_bf16x2(v.z, v.w));
+    }
+  }
+}
+
+extern "C" int rb_outnorm_residual(float* x, const float* a, const float* b, float sa, float sb, const float* gain, float eps,
+                                   int assign, void* h_out, int h_dtype, int n_tokens, int width, void* stream) {
+  RB_RECORDED(rb_outnorm_residual(x, a, b, sa, sb, gain, eps, assign, h_out, h_dtype, n_tokens, width, stream));
+  RB_REQUIRE(n_tokens >= 0 && width > 0, "rb_outnorm_residual: bad sizes %d x %d", n_tokens, width);
+  RB_REQUIRE(x && a && gain, "rb_outnorm_residual: the stream, the term and the gain are needed");
+  RB_REQUIRE(h_dtype == RB_F32 || h_dtype == RB_BF16, "rb_outnorm_residual: unknown dtype %d", h_dtype);
+  if (n_tokens == 0) return 0;
+  hipStream_t s = (hipStream_t)stream;
+  auto aligned = [](const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; };
+  if (width % 4 == 0 && aligned(x) && aligned(a) && aligned(b) && aligned(gain) && aligned(h_out)) {
+    int threads = ((width / 4 + RB_WAVE - 1) / RB_WAVE) * RB_WAVE;
+    if (threads > 1024) threads = 1024;
+    if (h_dtype == RB_F32)
+      outnorm_residual_vec_kernel<float><<<n_tokens, threads, 0, s>>>(x, a, b, sa, sb, gain, eps, assign, (float*)h_out, width);
+    else
+      outnorm_residual_vec_kernel<bf16_t><<<n_tokens, threads, 0, s>>>(x, a, b, sa, sb, gain, eps, assign, (bf16_t*)h_out, width);
+  } else {
+    const int threads = width >= 1024 ? 1024 : (width >= 256 ? 256 : 64);
+    if (h_dtype == RB_F32)
+      outnorm_residual_kernel<float><<<n_tokens, threads, 0, s>>>(x, a, b, sa, sb, gain, eps, assign, (float*)h_out, width);
+    else
+      outnorm_residual_kernel<bf16_t><<<n_tokens, threads, 0, s>>>(x, a, b, sa, sb, gain, eps, assign, (bf16_t*)h_out, width);
+  }
+  RB_LAUNCH_CHECK();
+  return 0;
+}
+
+// ---------------------------------------------------------------- a gated unit with limits
+// g = min(gu[r, j], limit), u = clamp(gu[r, F + j], -limit, limit); out[r, j] = g * sigmoid(alpha * g) * (u + 1).
+// limit <= 0: no limits.  Rows of gu are 2 F float32 numbers.
+template <typename TO>
+__global__ void clamped_glu_kernel(const float* __restrict__ gu, TO* __restrict__ out, int ff, float limit, float alpha,
+                                   size_t n) {
+  for (size_t e = (size_t)blockIdx.x * blockDim.x + threadIdx.x; e < n; e += (size_t)gridDim.x * blockDim.x) {
+    const size_t r = e / ff;
+    const int j = (int)(e - r * ff);
+    float g = gu[r * 2 * ff + j], u = gu[r * 2 * ff + ff + j];
+    if (limit > 0.f) {
+      g = fminf(g, limit);
+      u = fminf(fmaxf(u, -limit), limit);
+    }
+    Num<TO>::store(out + e, g / (1.0f + expf(-alpha * g)) * (u + 1.0f));
+  }
+}
+
+extern "C" int rb_clamped_glu(const float* gu, void* out, int out_dtype, int n_rows, int ff, float limit, float alpha,
+                              void* stream) {
+  RB_RECORDED(rb_clamped_glu(gu, out, out_dtype, n_rows, ff, limit, alpha, stream));
+  RB_REQUIRE(n_rows >= 0 && ff > 0, "rb_clamped_glu: bad sizes %d x %d", n_rows, ff);
+  if (n_rows == 0) return 0;
+  const size_t n = (size_t)n_rows * ff;
+  const size_t blocks = (n + 255) / 256;
+  const int grid = (int)(blocks < 65535 ? blocks : 65535);
+  hipStream_t s = (hipStream_t)stream;
+  if (out_dtype == RB_F32)
+    clamped_glu_kernel<float><<<grid, 256, 0, s>>>(gu, (float*)out, ff, limit, alpha, n);
+  else if (out_dtype == RB_BF16)
+    clamped_glu_kernel<bf16_t><<<grid, 256, 0, s>>>(gu, (bf16_t*)out, ff, limit, alpha, n);
+  else
+    RB_REQUIRE(false, "rb_clamped_glu: unknown dtype %d", out_dtype);
+  RB_LAUNCH_CHECK();
+  return 0;
+}
+
+// ---------------------------------------------------------------- tanh on the way to the compute dtype
+template <typename TO>
+__global__ void tanh_cast_kernel(const float* __restrict__ z, TO* __restrict__ out, size_t n) {
+  for (size_t e = (size_t)blockIdx.x * blockDim.x + threadIdx.x; e < n; e += (size_t)gridDim.x * blockDim.x)
+    Num<TO>::store(out + e, tanhf(z[e]));
+}
+
+extern "C" int rb_tanh_cast(const float* z, void* out, int out_dtype, long long n, void* stream) {
+  RB_RECORDED(rb_tanh_cast(z, out, out_dtype, n, stream));
+  RB_REQUIRE(n >= 0, "rb_tanh_cast: bad size");
+  if (n == 0) return 0;
+  const size_t blocks = ((size_t)n + 255) / 256;
+  const int grid = (int)(blocks < 65535 ? blocks : 65535);
+  hipStream_t s = (hipStream_t)stream;
+  if (out_dtype == RB_F32)
+    tanh_cast_kernel<float><<<grid, 256, 0, s>>>(z, (float*)out, (size_t)n);
+  else if (out_dtype == RB_BF16)
+    tanh_cast_kernel<bf16_t><<<grid, 256, 0, s>>>(z, (bf16_t*)out, (size_t)n);
+  else
+    RB_REQUIRE(false, "rb_tanh_cast: unknown dtype %d", out_dtype);
+  RB_LAUNCH_CHECK();
+  return 0;
+}

@@ -15,7 +15,7 @@
 template <typename TC>
 __global__ void latent_norm_store_kernel(const float* __restrict__ proj, size_t stride, int q_rank,
                                          const float* __restrict__ q_gain, TC* __restrict__ cq, int kv_col, int kv_rank,
-                                         const float* __restrict__ kv_gain, TC* __restrict__ pages,
+                                         const float* __restrict__ kv_gain, TC* __restrict__ pages, int page_width,
                                          const int32_t* __restrict__ tok_pos, const int32_t* __restrict__ tok_seq,
                                          const int32_t* __restrict__ block_table, int bt_stride, float eps) {
   __shared__ float scratch[16];
@@ -30,7 +30,7 @@ __global__ void latent_norm_store_kernel(const float* __restrict__ proj, size_t 
   if (kv_rank > 0) {
     const int pos = tok_pos[t];
     const int page = block_table[(size_t)tok_seq[t] * bt_stride + pos / RB_PAGE];
-    TC* dst = pages + ((size_t)page * RB_PAGE + (size_t)(pos % RB_PAGE)) * kv_rank;
+    TC* dst = pages + ((size_t)page * RB_PAGE + (size_t)(pos % RB_PAGE)) * page_width;
     const float* src = row + kv_col;
     float ss = 0.f;
     for (int j = threadIdx.x; j < kv_rank; j += blockDim.x) ss = fmaf(src[j], src[j], ss);
@@ -52,10 +52,10 @@ extern "C" int rb_latent_norm_store(const float* proj, long long stride, int q_r
   hipStream_t s = (hipStream_t)stream;
   if (dtype == RB_F32)
     latent_norm_store_kernel<float><<<n_tokens, 256, 0, s>>>(proj, (size_t)stride, q_rank, q_gain, (float*)cq, kv_col, kv_rank,
-                                                             kv_gain, (float*)pages, tok_pos, tok_seq, block_table, bt_stride, eps);
+                                                             kv_gain, (float*)pages, kv_rank, tok_pos, tok_seq, block_table, bt_stride, eps);
   else if (dtype == RB_BF16)
     latent_norm_store_kernel<bf16_t><<<n_tokens, 256, 0, s>>>(proj, (size_t)stride, q_rank, q_gain, (bf16_t*)cq, kv_col, kv_rank,
-                                                              kv_gain, (bf16_t*)pages, tok_pos, tok_seq, block_table, bt_stride, eps);
+                                                              kv_gain, (bf16_t*)pages, kv_rank, tok_pos, tok_seq, block_table, bt_stride, eps);
   else
     RB_REQUIRE(false, "rb_latent_norm_store: unknown dtype %d", dtype);
   RB_LAUNCH_CHECK();
@@ -72,7 +72,8 @@ extern "C" int rb_latent_norm_store(const float* proj, long long stride, int q_r
 #define HL_WAVES 4
 template <typename TX, typename TW, typename TY>
 __global__ __launch_bounds__(RB_WAVE * HL_WAVES) void heads_linear_kernel(const TX* __restrict__ x, const TW* __restrict__ w,
-                                                                          TY* __restrict__ y, int n_tokens, int n_heads, int n, int k) {
+                                                                          TY* __restrict__ y, int n_tokens, int n_heads, int n, int k,
+                                                                          size_t x_hs, size_t y_hs) {
   extern __shared__ float xs[];                  // [HL_TOKENS][k], then [HL_WAVES - 1][HL_TOKENS][64] partial sums
   float* part = xs + HL_TOKENS * k;
   const int t0 = blockIdx.x * HL_TOKENS, h = blockIdx.y;
@@ -85,7 +86,7 @@ __global__ __launch_bounds__(RB_WAVE * HL_WAVES) void heads_linear_kernel(const 
     for (int it = 0; it < 8; ++it) {
       const int idx = base + it * RB_WAVE * HL_WAVES + threadIdx.x;
       const int tt = idx / k, kk = idx - tt * k;
-      v[it] = (idx < HL_TOKENS * k && tt < nt) ? Num<TX>::load(x + ((size_t)(t0 + tt) * n_heads + h) * k + kk) : 0.f;
+      v[it] = (idx < HL_TOKENS * k && tt < nt) ? Num<TX>::load(x + ((size_t)(t0 + tt) * n_heads + h) * x_hs + kk) : 0.f;
     }
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
@@ -128,33 +129,163 @@ __global__ __launch_bounds__(RB_WAVE * HL_WAVES) void heads_linear_kernel(const 
     float v = acc[tt];
 #pragma unroll
     for (int ww = 0; ww < HL_WAVES - 1; ++ww) v += part[(ww * HL_TOKENS + tt) * RB_WAVE + lane];
-    if (tt < nt) Num<TY>::store(y + ((size_t)(t0 + tt) * n_heads + h) * n + col, v);
+    if (tt < nt) Num<TY>::store(y + ((size_t)(t0 + tt) * n_heads + h) * y_hs + col, v);
   }
 }
 
 template <typename TX, typename TW, typename TY>
-static void launch_heads_linear(const void* x, const void* w, void* y, int n_tokens, int n_heads, int n, int k, hipStream_t s) {
+static void launch_heads_linear(const void* x, const void* w, void* y, int n_tokens, int n_heads, int n, int k, size_t x_hs,
+                                size_t y_hs, hipStream_t s) {
   dim3 grid((n_tokens + HL_TOKENS - 1) / HL_TOKENS, n_heads, (n + RB_WAVE - 1) / RB_WAVE);
   const size_t lds = ((size_t)HL_TOKENS * k + (size_t)(HL_WAVES - 1) * HL_TOKENS * RB_WAVE) * sizeof(float);
-  heads_linear_kernel<TX, TW, TY><<<grid, RB_WAVE * HL_WAVES, lds, s>>>((const TX*)x, (const TW*)w, (TY*)y, n_tokens, n_heads, n, k);
+  heads_linear_kernel<TX, TW, TY><<<grid, RB_WAVE * HL_WAVES, lds, s>>>((const TX*)x, (const TW*)w, (TY*)y, n_tokens, n_heads, n, k, x_hs, y_hs);
 }
 
 extern "C" int rb_heads_linear(const void* x, int x_dtype, const void* w, int w_dtype, void* y, int y_dtype, int n_tokens,
                                int n_heads, int n, int k, void* stream) {
   RB_RECORDED(rb_heads_linear(x, x_dtype, w, w_dtype, y, y_dtype, n_tokens, n_heads, n, k, stream));
+  return rb_heads_linear_strided(x, x_dtype, k, w, w_dtype, y, y_dtype, n, n_tokens, n_heads, n, k, stream);
+}
+
+// The same with a head of x taking x_head_stride numbers (the first k of them are read) and a head of y y_head_stride
+// (the first n are written): products on a part of every head, into a part of every head.
+extern "C" int rb_heads_linear_strided(const void* x, int x_dtype, long long x_head_stride, const void* w, int w_dtype, void* y,
+                                       int y_dtype, long long y_head_stride, int n_tokens, int n_heads, int n, int k, void* stream) {
+  RB_RECORDED(rb_heads_linear_strided(x, x_dtype, x_head_stride, w, w_dtype, y, y_dtype, y_head_stride, n_tokens, n_heads, n, k,
+                                      stream));
   RB_REQUIRE(n_tokens >= 0 && n_heads > 0 && n_heads <= 65535 && n > 0 && n <= 65535 * 64 && k > 0, "rb_heads_linear: bad sizes");
   RB_REQUIRE(k <= 768, "rb_heads_linear: inner size %d not supported (at most 768)", k);
+  RB_REQUIRE(x_head_stride >= k && y_head_stride >= n, "rb_heads_linear: a head's stride is shorter than the head");
   if (n_tokens == 0) return 0;
   hipStream_t s = (hipStream_t)stream;
+  const size_t xs = (size_t)x_head_stride, ys = (size_t)y_head_stride;
   const int key = x_dtype * 4 + w_dtype * 2 + y_dtype;
   switch (key) {
-    case 0: launch_heads_linear<float, float, float>(x, w, y, n_tokens, n_heads, n, k, s); break;
-    case 3: launch_heads_linear<float, bf16_t, bf16_t>(x, w, y, n_tokens, n_heads, n, k, s); break;
-    case 6: launch_heads_linear<bf16_t, bf16_t, float>(x, w, y, n_tokens, n_heads, n, k, s); break;
-    case 7: launch_heads_linear<bf16_t, bf16_t, bf16_t>(x, w, y, n_tokens, n_heads, n, k, s); break;
-    case 2: launch_heads_linear<float, bf16_t, float>(x, w, y, n_tokens, n_heads, n, k, s); break;
+    case 0: launch_heads_linear<float, float, float>(x, w, y, n_tokens, n_heads, n, k, xs, ys, s); break;
+    case 3: launch_heads_linear<float, bf16_t, bf16_t>(x, w, y, n_tokens, n_heads, n, k, xs, ys, s); break;
+    case 6: launch_heads_linear<bf16_t, bf16_t, float>(x, w, y, n_tokens, n_heads, n, k, xs, ys, s); break;
+    case 7: launch_heads_linear<bf16_t, bf16_t, bf16_t>(x, w, y, n_tokens, n_heads, n, k, xs, ys, s); break;
+    case 2: launch_heads_linear<float, bf16_t, float>(x, w, y, n_tokens, n_heads, n, k, xs, ys, s); break;
     default: RB_REQUIRE(false, "rb_heads_linear: this combination of types is not built (x %d, w %d, y %d)", x_dtype, w_dtype, y_dtype);
   }
+  RB_LAUNCH_CHECK();
+  return 0;
+}
+
+// ---------------------------------------------------------------- a rotated part beside the latent
+// Where a head's key is a part made from the latent beside a rotated part that all heads share, the cache holds per token
+// the latent c and, behind it, that rotated part: one key/value head of page_width >= kv_rank + rot numbers (the rest
+// zeros), and a query is [Wk^T q_unrotated, rotate(q_rotated)] in the same layout.
+// rb_latent_norm_store with that: the `rot` numbers at rot_col of a row of proj are rotated by the token's position
+// (style 0: 2i with 2i + 1; 1: i with i + rot / 2; cos, sin [positions, rot / 2]) and stored behind the latent.
+template <typename TC>
+__global__ void latent_rope_store_kernel(const float* __restrict__ proj, size_t stride, int kv_rank, int page_width, int rot_col,
+                                         int rot, const float* __restrict__ cos_t, const float* __restrict__ sin_t, int style,
+                                         TC* __restrict__ pages, const int32_t* __restrict__ tok_pos,
+                                         const int32_t* __restrict__ tok_seq, const int32_t* __restrict__ block_table, int bt_stride) {
+  const int t = blockIdx.x;
+  const int pos = tok_pos[t];
+  const int half = rot / 2;
+  const int page = block_table[(size_t)tok_seq[t] * bt_stride + pos / RB_PAGE];
+  TC* dst = pages + ((size_t)page * RB_PAGE + (size_t)(pos % RB_PAGE)) * page_width + kv_rank;
+  const float* src = proj + (size_t)t * stride + rot_col;
+  const float* cr = cos_t + (size_t)pos * half;
+  const float* sr = sin_t + (size_t)pos * half;
+  for (int i = threadIdx.x; i < half; i += blockDim.x) {
+    const int a = style == 0 ? 2 * i : i, b = style == 0 ? 2 * i + 1 : i + half;
+    float y0, y1;
+    rotate_pair(src[a], src[b], cr[i], sr[i], y0, y1);
+    Num<TC>::store(dst + a, y0);
+    Num<TC>::store(dst + b, y1);
+  }
+  for (int i = rot + threadIdx.x; i < page_width - kv_rank; i += blockDim.x) Num<TC>::store(dst + i, 0.f);
+}
+
+extern "C" int rb_latent_norm_rope_store(const float* proj, long long stride, int q_rank, const float* q_gain, void* cq, int kv_col,
+                                         int kv_rank, const float* kv_gain, void* pages, int page_width, int rot_col, int rot,
+                                         const float* cos, const float* sin, int style, int dtype, const int32_t* tok_pos,
+                                         const int32_t* tok_seq, const int32_t* block_table, int bt_stride, float eps, int n_tokens,
+                                         void* stream) {
+  RB_RECORDED(rb_latent_norm_rope_store(proj, stride, q_rank, q_gain, cq, kv_col, kv_rank, kv_gain, pages, page_width, rot_col, rot,
+                                        cos, sin, style, dtype, tok_pos, tok_seq, block_table, bt_stride, eps, n_tokens, stream));
+  RB_REQUIRE(n_tokens >= 0 && q_rank >= 0 && kv_rank >= 0 && kv_col >= 0 && rot >= 0 && rot % 2 == 0 && rot_col >= 0,
+             "rb_latent_norm_rope_store: bad sizes");
+  RB_REQUIRE(stride >= q_rank && stride >= (long long)kv_col + kv_rank && stride >= (long long)rot_col + rot,
+             "rb_latent_norm_rope_store: the row stride is too short");
+  RB_REQUIRE(kv_rank == 0 || (pages && block_table && page_width >= kv_rank + rot),
+             "rb_latent_norm_rope_store: a latent needs cache pages that hold it and the rotated part");
+  RB_REQUIRE(rot == 0 || kv_rank == 0 || (cos && sin && (style == 0 || style == 1)), "rb_latent_norm_rope_store: a rotation needs its tables");
+  RB_REQUIRE(dtype == RB_F32 || dtype == RB_BF16, "rb_latent_norm_rope_store: unknown dtype %d", dtype);
+  if (n_tokens == 0) return 0;
+  hipStream_t s = (hipStream_t)stream;
+  if (dtype == RB_F32)
+    latent_norm_store_kernel<float><<<n_tokens, 256, 0, s>>>(proj, (size_t)stride, q_rank, q_gain, (float*)cq, kv_col, kv_rank,
+                                                             kv_gain, (float*)pages, page_width, tok_pos, tok_seq, block_table,
+                                                             bt_stride, eps);
+  else
+    latent_norm_store_kernel<bf16_t><<<n_tokens, 256, 0, s>>>(proj, (size_t)stride, q_rank, q_gain, (bf16_t*)cq, kv_col, kv_rank,
+                                                              kv_gain, (bf16_t*)pages, page_width, tok_pos, tok_seq, block_table,
+                                                              bt_stride, eps);
+  if (kv_rank > 0 && page_width > kv_rank) {
+    if (dtype == RB_F32)
+      latent_rope_store_kernel<float><<<n_tokens, 64, 0, s>>>(proj, (size_t)stride, kv_rank, page_width, rot_col, rot, cos, sin,
+                                                              style, (float*)pages, tok_pos, tok_seq, block_table, bt_stride);
+    else
+      latent_rope_store_kernel<bf16_t><<<n_tokens, 64, 0, s>>>(proj, (size_t)stride, kv_rank, page_width, rot_col, rot, cos, sin,
+                                                               style, (bf16_t*)pages, tok_pos, tok_seq, block_table, bt_stride);
+  }
+  RB_LAUNCH_CHECK();
+  return 0;
+}
+
+// The queries' side of the same: of every head of x [T, H, x_head_stride] float32 the `rot` numbers at x_col are rotated by the
+// token's position and written to y [T, H, y_head_stride] at y_col; what lies behind them up to y_head_stride becomes zero.
+template <typename TC>
+__global__ void rope_heads_part_kernel(const float* __restrict__ x, size_t x_hs, int x_col, int rot, const float* __restrict__ cos_t,
+                                       const float* __restrict__ sin_t, int style, TC* __restrict__ y, size_t y_hs, int y_col,
+                                       const int32_t* __restrict__ tok_pos, int n_heads) {
+  const int t = blockIdx.x;
+  const int pos = tok_pos[t];
+  const int half = rot / 2;
+  const float* cr = cos_t + (size_t)pos * half;
+  const float* sr = sin_t + (size_t)pos * half;
+  const int tail = (int)y_hs - y_col - rot;
+  const int per_head = half + tail;
+  for (int idx = threadIdx.x; idx < n_heads * per_head; idx += blockDim.x) {
+    const int h = idx / per_head, i = idx - h * per_head;
+    const float* src = x + ((size_t)t * n_heads + h) * x_hs + x_col;
+    TC* dst = y + ((size_t)t * n_heads + h) * y_hs + y_col;
+    if (i < half) {
+      const int a = style == 0 ? 2 * i : i, b = style == 0 ? 2 * i + 1 : i + half;
+      float y0, y1;
+      rotate_pair(src[a], src[b], cr[i], sr[i], y0, y1);
+      Num<TC>::store(dst + a, y0);
+      Num<TC>::store(dst + b, y1);
+    } else {
+      Num<TC>::store(dst + rot + (i - half), 0.f);
+    }
+  }
+}
+
+extern "C" int rb_rope_heads_part(const float* x, long long x_head_stride, int x_col, int rot, const float* cos, const float* sin,
+                                  int style, void* y, int y_dtype, long long y_head_stride, int y_col, const int32_t* tok_pos,
+                                  int n_tokens, int n_heads, void* stream) {
+  RB_RECORDED(rb_rope_heads_part(x, x_head_stride, x_col, rot, cos, sin, style, y, y_dtype, y_head_stride, y_col, tok_pos, n_tokens,
+                                 n_heads, stream));
+  RB_REQUIRE(n_tokens >= 0 && n_heads > 0 && rot >= 0 && rot % 2 == 0 && x_col >= 0 && y_col >= 0, "rb_rope_heads_part: bad sizes");
+  RB_REQUIRE(x_head_stride >= (long long)x_col + rot && y_head_stride >= (long long)y_col + rot,
+             "rb_rope_heads_part: the rotated part lies outside a head");
+  RB_REQUIRE(rot == 0 || (cos && sin && (style == 0 || style == 1)), "rb_rope_heads_part: a rotation needs its tables");
+  if (n_tokens == 0 || y_head_stride == y_col) return 0;
+  hipStream_t s = (hipStream_t)stream;
+  if (y_dtype == RB_F32)
+    rope_heads_part_kernel<float><<<n_tokens, 256, 0, s>>>(x, (size_t)x_head_stride, x_col, rot, cos, sin, style, (float*)y,
+                                                           (size_t)y_head_stride, y_col, tok_pos, n_heads);
+  else if (y_dtype == RB_BF16)
+    rope_heads_part_kernel<bf16_t><<<n_tokens, 256, 0, s>>>(x, (size_t)x_head_stride, x_col, rot, cos, sin, style, (bf16_t*)y,
+                                                            (size_t)y_head_stride, y_col, tok_pos, n_heads);
+  else
+    RB_REQUIRE(false, "rb_rope_heads_part: unknown dtype %d", y_dtype);
   RB_LAUNCH_CHECK();
   return 0;
 }

@@ -105,7 +105,7 @@ class KernelTimes:
         return "\n".join(lines)
 
 
-TIMED_OPS = ("route_choose", "experts_combine", "embed_scaled_pos", "scale", "bias_norm_store", "attention_mixed", "attention_mixed_bf16", "recurrence_prep", "linear_recurrence", "layernorm_residual", "rope_store", "head_gate", "pair_norm_mean",
+TIMED_OPS = ("outnorm_residual", "clamped_glu", "tanh_cast", "attention_opts", "norm_rope_store", "sigmoid_gate", "shift_mix", "time_mix_recurrence", "latent_norm_rope_store", "rope_heads_part", "heads_linear_part", "route_choose", "experts_combine", "embed_scaled_pos", "scale", "bias_norm_store", "attention_mixed", "attention_mixed_bf16", "recurrence_prep", "linear_recurrence", "layernorm_residual", "rope_store", "head_gate", "pair_norm_mean",
              "route_top", "routed_experts", "pairs_sum", "embed_streams", "streams_layernorm", "streams_update", "xielu", "tanh_cap", "short_conv",
              "delta_prep", "delta_rule", "gated_rmsnorm", "latent_norm_store", "heads_linear", "attention_sinks", "embed_gather", "add_rmsnorm", "rope_kv_write", "swiglu", "gemm_generic", "gemm_bf16", "gemm_bf16_terms",
              "gemm_bf16_few", "attention_generic", "attention_prefill_bf16", "attention_decode_bf16",
@@ -181,6 +181,19 @@ class Kernels:
             "rb_embed_scaled_pos": [_P, _I, _P, _F, _P, _P, _P, _I, _I, _P],
             "rb_scale": [_P, _F, _L, _P],
             "rb_bias_norm_store": [_P, _L, _P, _I, _F, _P, _P, _P, _I, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _P],
+            "rb_outnorm_residual": [_P, _P, _P, _F, _F, _P, _F, _I, _P, _I, _I, _I, _P],
+            "rb_clamped_glu": [_P, _P, _I, _I, _I, _F, _F, _P],
+            "rb_tanh_cast": [_P, _P, _I, _L, _P],
+            "rb_attention_generic_opts": [_P, _P, _P, _P, _I, _P, _P, _P, _I, _I, _I, _I, _I, _F, _I, _I, _F, _P, _P],
+            "rb_norm_rope_store": [_P, _L, _P, _P, _I, _P, _P, _F, _P, _P, _P, _I, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _P],
+            "rb_sigmoid_gate": [_P, _I, _P, _L, _P],
+            "rb_shift_mix": [_P, _I, _P, _P, _I, _P, _P, _P, _P, _I, _I, _I, _P],
+            "rb_short_conv_bias": [_P, _L, _P, _P, _I, _P, _P, _P, _P, _P, _P, _L, _I, _I, _I, _I, _I, _I, _P],
+            "rb_linear_recurrence_bonus": [_P, _P, _L, _P, _L, _P, _L, _I, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P],
+            "rb_gated_rmsnorm_heads": [_P, _P, _L, _P, _L, _I, _F, _P, _I, _I, _I, _I, _P],
+            "rb_heads_linear_strided": [_P, _I, _L, _P, _I, _P, _I, _L, _I, _I, _I, _I, _P],
+            "rb_latent_norm_rope_store": [_P, _L, _I, _P, _P, _I, _I, _P, _P, _I, _I, _I, _P, _P, _I, _I, _P, _P, _P, _I, _F, _I, _P],
+            "rb_rope_heads_part": [_P, _L, _I, _I, _P, _P, _I, _P, _I, _L, _I, _P, _I, _I, _P],
             "rb_attention_mixed": [_P, _P, _P, _P, _I, _P, _P, _P, _I, _I, _I, _I, _I, _F, _P, _I, _I, _P],
             "rb_attention_mixed_bf16": [_P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _P, _I, _I, _I, _P, _P],
         }
@@ -1000,6 +1013,230 @@ class Kernels:
                                                       _ptr(tok_pos), _ptr(tok_seq), _ptr(block_table), block_table.shape[1],
                                                       n, n_heads, n_kv, head_dim, float(scale), int(window or 0),
                                                       _ptr(sinks), self._stream()))
+
+    # ------------------------------------------------------------------ layers with the norm on the sublayer's output
+    def outnorm_residual(self, x: torch.Tensor, a: torch.Tensor, b: Optional[torch.Tensor], sa: float, sb: float,
+                         gain: torch.Tensor, eps: float, assign: bool, h_out: Optional[torch.Tensor]) -> None:
+        """x [T, E] float32 <- (assign ? 0 : x) + rmsnorm(sa a + sb b) * gain; h_out [T, E] gets the new rows in its dtype."""
+        n, width = x.shape
+        _check(x, "x", torch.float32)
+        _check(a, "a", torch.float32, (n, width))
+        if b is not None:
+            _check(b, "b", torch.float32, (n, width))
+        _check(gain, "gain", torch.float32, (width,))
+        if h_out is not None:
+            _check(h_out, "h_out", None, (n, width))
+        self._ok(self._lib.rb_outnorm_residual(_ptr(x), _ptr(a), _ptr(b), float(sa), float(sb), _ptr(gain), float(eps),
+                                               int(bool(assign)), _ptr(h_out), dtype_code(h_out.dtype) if h_out is not None else _F32,
+                                               n, width, self._stream()))
+
+    def clamped_glu(self, gu: torch.Tensor, out: torch.Tensor, limit: float, alpha: float) -> None:
+        """gu [T, 2 F] float32 (gate, then up) -> out [T, F] = g sigmoid(alpha g) (u + 1) with g, u limited."""
+        n, ff = out.shape
+        _check(gu, "gu", torch.float32, (n, 2 * ff))
+        _check(out, "out")
+        self._ok(self._lib.rb_clamped_glu(_ptr(gu), _ptr(out), dtype_code(out.dtype), n, ff, float(limit), float(alpha), self._stream()))
+
+    def tanh_cast(self, z: torch.Tensor, out: torch.Tensor) -> None:
+        _check(z, "z", torch.float32)
+        _check(out, "out", None, z.shape)
+        self._ok(self._lib.rb_tanh_cast(_ptr(z), _ptr(out), dtype_code(out.dtype), z.numel(), self._stream()))
+
+    def attention_opts(self, q, k_pages, v_pages, out, tok_pos, tok_seq, block_table, n_heads, n_kv, head_dim, scale, window,
+                       keep_first, softcap, sinks) -> None:
+        """`attention_sinks` with kept first keys behind the window and capped scores."""
+        n = q.shape[0]
+        _check(q, "q", None, (n, n_heads, head_dim))
+        _check(k_pages, "k_pages", q.dtype)
+        _check(v_pages, "v_pages", q.dtype, k_pages.shape)
+        if tuple(k_pages.shape[1:]) != (n_kv, self.page_size, head_dim):
+            raise KernelError("cache pages do not match the head counts")
+        _check(out, "out", q.dtype, (n, n_heads * head_dim))
+        _check(tok_pos, "tok_pos", torch.int32, (n,))
+        _check(tok_seq, "tok_seq", torch.int32, (n,))
+        _check(block_table, "block_table", torch.int32)
+        if sinks is not None:
+            _check(sinks, "sinks", torch.float32, (n_heads,))
+        self._ok(self._lib.rb_attention_generic_opts(_ptr(q), _ptr(k_pages), _ptr(v_pages), _ptr(out), dtype_code(q.dtype),
+                                                     _ptr(tok_pos), _ptr(tok_seq), _ptr(block_table), block_table.shape[1],
+                                                     n, n_heads, n_kv, head_dim, float(scale), int(window or 0),
+                                                     int(keep_first or 0), float(softcap or 0.0), _ptr(sinks), self._stream()))
+
+    def norm_rope_store(self, qkv: torch.Tensor, cos, sin, rot: int, q_norm: torch.Tensor, k_norm: Optional[torch.Tensor], eps: float,
+                        q_out: torch.Tensor, k_pages, v_pages, tok_pos, tok_seq, block_table, n_heads: int, n_kv: int, dim: int,
+                        vdim: int, pad: int) -> None:
+        """`rope_store` with every query and key head RMS-normed first (weights float32 [dim])."""
+        n, width = qkv.shape
+        _check(qkv, "qkv", torch.float32)
+        _check(q_out, "q_out", None, (n, n_heads, pad))
+        _check(tok_pos, "tok_pos", torch.int32, (n,))
+        _check(tok_seq, "tok_seq", torch.int32, (n,))
+        _check(q_norm, "q_norm", torch.float32, (dim,))
+        if rot:
+            _check(cos, "cos", torch.float32)
+            _check(sin, "sin", torch.float32, cos.shape)
+            if cos.shape[1] != rot // 2:
+                raise KernelError("angle table width mismatch")
+        need = n_heads * dim
+        if k_pages is not None:
+            need += n_kv * (dim + vdim)
+            _check(k_norm, "k_norm", torch.float32, (dim,))
+            _check(block_table, "block_table", torch.int32)
+            _check(k_pages, "k_pages", q_out.dtype)
+            _check(v_pages, "v_pages", q_out.dtype, k_pages.shape)
+            if tuple(k_pages.shape[1:]) != (n_kv, self.page_size, pad):
+                raise KernelError(f"cache pages have shape {tuple(k_pages.shape)}, expected [*, {n_kv}, {self.page_size}, {pad}]")
+        if width < need:
+            raise KernelError("norm_rope_store: rows too short for the heads")
+        self._ok(self._lib.rb_norm_rope_store(_ptr(qkv), width, _ptr(cos) if rot else None, _ptr(sin) if rot else None, int(rot),
+                                              _ptr(q_norm), _ptr(k_norm), float(eps), _ptr(q_out), _ptr(k_pages), _ptr(v_pages),
+                                              dtype_code(q_out.dtype), _ptr(tok_pos), _ptr(tok_seq),
+                                              _ptr(block_table) if k_pages is not None else None,
+                                              block_table.shape[1] if k_pages is not None else 0, n, n_heads,
+                                              n_kv if k_pages is not None else 0, dim, vdim, pad, self._stream()))
+
+    def sigmoid_gate(self, x: torch.Tensor, gate: torch.Tensor) -> None:
+        """x *= sigmoid(gate), in place; both [T, N], gate float32."""
+        _check(x, "x")
+        _check(gate, "gate", torch.float32, x.shape)
+        self._ok(self._lib.rb_sigmoid_gate(_ptr(x), dtype_code(x.dtype), _ptr(gate), x.numel(), self._stream()))
+
+    def shift_mix(self, h: torch.Tensor, state: torch.Tensor, mu: torch.Tensor, ctx, out: torch.Tensor) -> None:
+        """out[m] = h + (the row before - h) * mu[m]; state [slots, E] float32 holds every sequence's last row."""
+        n, width = h.shape
+        m = mu.shape[0]
+        _check(h, "h")
+        _check(mu, "mu", torch.float32, (m, width))
+        _check(state, "state", torch.float32)
+        if tuple(state.shape[1:]) != (width,):
+            raise KernelError(f"shift_mix: state of shape {tuple(state.shape)}, expected [*, {width}]")
+        _check(out, "out", h.dtype, (m, n, width))
+        if ctx.n_tokens != n:
+            raise KernelError("shift_mix: the step's tokens and the rows differ")
+        self._ok(self._lib.rb_shift_mix(_ptr(h), dtype_code(h.dtype), _ptr(state), _ptr(mu), m, _ptr(out), _ptr(ctx.cu_seqlens),
+                                        _ptr(ctx.tok_seq), _ptr(ctx.slots), n, ctx.n_seqs, width, self._stream()))
+
+    def short_conv_bias(self, x: torch.Tensor, col0: int, channels: int, bias: Optional[torch.Tensor], w: torch.Tensor,
+                        state: Optional[torch.Tensor], ctx, out: torch.Tensor, residual: bool, act: int) -> None:
+        """`short_conv` on x + bias (float32 [channels]); the state holds the inputs with their bias."""
+        n, width = x.shape
+        taps = w.shape[1]
+        _check(x, "x", torch.float32)
+        _check(w, "w", torch.float32, (channels, taps))
+        if bias is not None:
+            _check(bias, "bias", torch.float32, (channels,))
+        if col0 < 0 or col0 + channels > width:
+            raise KernelError("short_conv: the columns lie outside the rows")
+        if taps > 1:
+            _check(state, "state", torch.float32)
+            if tuple(state.shape[1:]) != (taps - 1, channels):
+                raise KernelError(f"short_conv: state of shape {tuple(state.shape)}, expected [*, {taps - 1}, {channels}]")
+        _check(out, "out", None, (n, channels))
+        _check(ctx.tok_pos, "tok_pos", torch.int32, (n,))
+        self._ok(self._lib.rb_short_conv_bias(x.data_ptr() + 4 * col0, width, _ptr(bias), _ptr(w), taps,
+                                              _ptr(state) if taps > 1 else None, _ptr(ctx.tok_pos), _ptr(ctx.tok_seq),
+                                              _ptr(ctx.cu_seqlens), _ptr(ctx.slots), _ptr(out), channels, dtype_code(out.dtype),
+                                              int(bool(residual)), int(act), n, ctx.n_seqs, channels, self._stream()))
+
+    def time_mix_recurrence(self, r: torch.Tensor, k: torch.Tensor, v: torch.Tensor, decay: torch.Tensor, bonus: torch.Tensor,
+                            state: torch.Tensor, ctx, out: torch.Tensor, n_heads: int, dim: int, vdim: int) -> None:
+        """r, k, decay [T, H dim], v [T, H vdim] float32; bonus [H, dim]; state [slots, H, vdim, dim] float32:
+        out = (S + diag(bonus) k v^T)^T r, then S <- diag(decay) S + k v^T, token after token."""
+        n = r.shape[0]
+        _check(r, "r", torch.float32, (n, n_heads * dim))
+        _check(k, "k", torch.float32, (n, n_heads * dim))
+        _check(v, "v", torch.float32, (n, n_heads * vdim))
+        _check(decay, "decay", torch.float32, (n, n_heads * dim))
+        _check(bonus, "bonus", torch.float32, (n_heads, dim))
+        _check(state, "state", torch.float32)
+        if tuple(state.shape[1:]) != (n_heads, vdim, dim):
+            raise KernelError(f"time_mix_recurrence: state of shape {tuple(state.shape)}, expected [*, {n_heads}, {vdim}, {dim}]")
+        _check(out, "out", torch.float32, (n, n_heads * vdim))
+        if ctx.n_tokens != n:
+            raise KernelError("time_mix_recurrence: the step's tokens and the rows differ")
+        self._ok(self._lib.rb_linear_recurrence_bonus(_ptr(r), _ptr(k), n_heads * dim, _ptr(v), n_heads * vdim, _ptr(decay),
+                                                      n_heads * dim, 0, None, _ptr(bonus), _ptr(state), _ptr(ctx.cu_seqlens),
+                                                      _ptr(ctx.slots), _ptr(out), ctx.n_seqs, n, n_heads, n_heads, dim, vdim,
+                                                      self._stream()))
+
+    def decay_exp_exp(self, z: torch.Tensor, bias: torch.Tensor, n_heads: int, dim: int) -> None:
+        """z [T, H dim] float32 <- exp(-exp(z + bias)), in place."""
+        n = z.shape[0]
+        _check(z, "z", torch.float32, (n, n_heads * dim))
+        _check(bias, "bias", torch.float32, (n_heads * dim,))
+        # the q and k heads are left as they are (no unit vectors, a scale of one): any valid rows serve
+        self._ok(self._lib.rb_recurrence_prep(_ptr(z), n_heads * dim, 0, dim, 0, 1.0, 0.0, _ptr(z), n_heads * dim, n_heads * dim, 2,
+                                              _ptr(bias), None, 1.0, n_heads, None, 0, None, n, self._stream()))
+
+    def gated_rmsnorm_heads(self, o: torch.Tensor, weight: torch.Tensor, gate: torch.Tensor, act: int, eps: float, n_heads: int,
+                            vdim: int, out: torch.Tensor) -> None:
+        """`gated_rmsnorm_act` with a weight over the concatenated heads [H * vdim]; gate [T, H * vdim] float32."""
+        n = o.shape[0]
+        _check(o, "o", torch.float32, (n, n_heads * vdim))
+        _check(weight, "weight", torch.float32, (n_heads * vdim,))
+        _check(gate, "gate", torch.float32, (n, n_heads * vdim))
+        _check(out, "out", None, (n, n_heads * vdim))
+        self._ok(self._lib.rb_gated_rmsnorm_heads(_ptr(o), _ptr(weight), vdim, _ptr(gate), n_heads * vdim, int(act), float(eps),
+                                                  _ptr(out), dtype_code(out.dtype), n, n_heads, vdim, self._stream()))
+
+    def heads_linear_part(self, x: torch.Tensor, x_head: int, w: torch.Tensor, y: torch.Tensor, y_head: int) -> None:
+        """y[t, h, :N] = w[h]^T x[t, h, :K] with w [H, K, N]; a head of x takes x_head numbers, a head of y y_head."""
+        h, k, n_out = w.shape
+        n = x.shape[0]
+        _check(x, "x", None, (n, h * x_head))
+        _check(w, "w")
+        _check(y, "y", None, (n, h * y_head))
+        if x_head < k or y_head < n_out:
+            raise KernelError("heads_linear_part: a head is shorter than the product's sizes")
+        self._ok(self._lib.rb_heads_linear_strided(_ptr(x), dtype_code(x.dtype), x_head, _ptr(w), dtype_code(w.dtype), _ptr(y),
+                                                   dtype_code(y.dtype), y_head, n, h, n_out, k, self._stream()))
+
+    def latent_norm_rope_store(self, proj: torch.Tensor, q_rank: int, q_gain, cq, kv_rank: int, kv_gain, pages, rot: int, cos, sin,
+                               style: int, ctx, block_table, eps: float, dtype: torch.dtype) -> None:
+        """proj [T, q_rank + kv_rank + rot] float32: cq [T, q_rank] and the pages [*, 1, 64, W >= kv_rank + rot] get the two RMS
+        norms, the pages also the last `rot` numbers rotated by the position, behind the latent, and zeros up to W."""
+        n, width = proj.shape
+        has_kv = kv_rank > 0
+        _check(proj, "proj", torch.float32, (n, q_rank + ((kv_rank + rot) if has_kv else 0)))
+        _check(q_gain, "q_gain", torch.float32, (q_rank,))
+        _check(cq, "cq", dtype, (n, q_rank))
+        page_width = 0
+        if has_kv:
+            _check(kv_gain, "kv_gain", torch.float32, (kv_rank,))
+            _check(pages, "pages", dtype)
+            page_width = pages.shape[-1]
+            if tuple(pages.shape[1:3]) != (1, self.page_size) or page_width < kv_rank + rot:
+                raise KernelError(f"latent pages have shape {tuple(pages.shape)}, expected [*, 1, {self.page_size}, >= {kv_rank + rot}]")
+            _check(block_table, "block_table", torch.int32)
+            if rot:
+                _check(cos, "cos", torch.float32)
+                _check(sin, "sin", torch.float32, cos.shape)
+                if cos.shape[1] != rot // 2:
+                    raise KernelError("angle table width mismatch")
+        self._ok(self._lib.rb_latent_norm_rope_store(_ptr(proj), width, q_rank, _ptr(q_gain), _ptr(cq), q_rank, kv_rank, _ptr(kv_gain),
+                                                     _ptr(pages) if has_kv else None, page_width, q_rank + kv_rank, rot if has_kv else 0,
+                                                     _ptr(cos) if rot else None, _ptr(sin) if rot else None, int(style),
+                                                     dtype_code(dtype), _ptr(ctx.tok_pos), _ptr(ctx.tok_seq),
+                                                     _ptr(block_table) if has_kv else None, block_table.shape[1] if has_kv else 0,
+                                                     float(eps), n, self._stream()))
+
+    def rope_heads_part(self, x: torch.Tensor, x_head: int, x_col: int, rot: int, cos, sin, style: int, y: torch.Tensor, y_head: int,
+                        y_col: int, tok_pos, n_heads: int) -> None:
+        """The `rot` numbers at x_col of every head of x [T, H * x_head] float32, rotated, to y [T, H * y_head] at y_col; zeros behind."""
+        n = x.shape[0]
+        _check(x, "x", torch.float32, (n, n_heads * x_head))
+        _check(y, "y", None, (n, n_heads * y_head))
+        _check(tok_pos, "tok_pos", torch.int32, (n,))
+        if x_col + rot > x_head or y_col + rot > y_head:
+            raise KernelError("rope_heads_part: the rotated part lies outside a head")
+        if rot:
+            _check(cos, "cos", torch.float32)
+            _check(sin, "sin", torch.float32, cos.shape)
+            if cos.shape[1] != rot // 2:
+                raise KernelError("angle table width mismatch")
+        self._ok(self._lib.rb_rope_heads_part(_ptr(x), x_head, x_col, rot, _ptr(cos) if rot else None, _ptr(sin) if rot else None,
+                                              int(style), _ptr(y), dtype_code(y.dtype), y_head, y_col, _ptr(tok_pos), n, n_heads,
+                                              self._stream()))
 
     # ------------------------------------------------------------------ recorded steps
     def plan_begin(self) -> int:

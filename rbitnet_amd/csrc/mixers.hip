@@ -293,3 +293,159 @@ extern "C" int rb_pair_norm_mean(const float* a, const float* wa, const float* b
   RB_LAUNCH_CHECK();
   return 0;
 }
+
+// ---------------------------------------------------------------- a norm per head in front of the rotation
+// rb_rope_store with every query and key head first RMS-normed over its `dim` numbers with a weight of that size shared by
+// the heads (q_norm, k_norm; plain weights): x / sqrt(mean(x^2) + eps) * w, in float32, then the rotation of the head's
+// first `rot` numbers, the padding and the cache write as there.  A wave takes a head.
+template <typename TC>
+__global__ void norm_rope_store_kernel(const float* __restrict__ qkv, size_t row_width, const float* __restrict__ cos_t,
+                                       const float* __restrict__ sin_t, int rot, const float* __restrict__ q_norm,
+                                       const float* __restrict__ k_norm, float eps, TC* __restrict__ q_out,
+                                       TC* __restrict__ k_pages, TC* __restrict__ v_pages, const int32_t* __restrict__ tok_pos,
+                                       const int32_t* __restrict__ tok_seq, const int32_t* __restrict__ block_table,
+                                       int bt_stride, int n_heads, int n_kv, int dim, int vdim, int pad) {
+  const int t = blockIdx.x;
+  const int pos = tok_pos[t];
+  const int half = rot / 2;
+  const int lane = threadIdx.x & (RB_WAVE - 1), wave = threadIdx.x / RB_WAVE, n_waves = blockDim.x / RB_WAVE;
+  const float* src = qkv + (size_t)t * row_width;
+  const float* cr = cos_t + (size_t)pos * half;
+  const float* sr = sin_t + (size_t)pos * half;
+  size_t page_base = 0;
+  if (k_pages) {
+    const int page = block_table[(size_t)tok_seq[t] * bt_stride + pos / RB_PAGE];
+    page_base = ((size_t)page * n_kv) * RB_PAGE * pad + (size_t)(pos % RB_PAGE) * pad;
+  }
+  const int n_rot_heads = n_heads + (k_pages ? n_kv : 0);
+  for (int h = wave; h < n_rot_heads; h += n_waves) {
+    const float* hp = src + (size_t)h * dim;
+    const float* w = h < n_heads ? q_norm : k_norm;
+    float ss = 0.f;
+    for (int d = lane; d < dim; d += RB_WAVE) ss = fmaf(hp[d], hp[d], ss);
+    const float f = 1.0f / sqrtf(wave_sum(ss) / (float)dim + eps);
+    TC* dst = h < n_heads ? q_out + ((size_t)t * n_heads + h) * pad
+                          : k_pages + page_base + (size_t)(h - n_heads) * RB_PAGE * pad;
+    for (int d = lane; d < pad; d += RB_WAVE) {
+      float y = 0.f;
+      if (d < half) {
+        float y1;
+        rotate_pair(hp[d] * f * w[d], hp[d + half] * f * w[d + half], cr[d], sr[d], y, y1);
+      } else if (d < rot) {
+        float y0;
+        rotate_pair(hp[d - half] * f * w[d - half], hp[d] * f * w[d], cr[d - half], sr[d - half], y0, y);
+      } else if (d < dim) {
+        y = hp[d] * f * w[d];
+      }
+      Num<TC>::store(dst + d, y);
+    }
+  }
+  if (v_pages) {
+    const float* vsrc = src + (size_t)(n_heads + n_kv) * dim;
+    for (int idx = threadIdx.x; idx < n_kv * pad; idx += blockDim.x) {
+      const int h = idx / pad, d = idx - h * pad;
+      Num<TC>::store(v_pages + page_base + (size_t)h * RB_PAGE * pad + d, d < vdim ? vsrc[(size_t)h * vdim + d] : 0.f);
+    }
+  }
+}
+
+extern "C" int rb_norm_rope_store(const float* qkv, long long row_width, const float* cos, const float* sin, int rot,
+                                  const float* q_norm, const float* k_norm, float eps, void* q_out, void* k_pages, void* v_pages,
+                                  int cache_dtype, const int32_t* tok_pos, const int32_t* tok_seq, const int32_t* block_table,
+                                  int bt_stride, int n_tokens, int n_heads, int n_kv_heads, int dim, int vdim, int pad,
+                                  void* stream) {
+  RB_RECORDED(rb_norm_rope_store(qkv, row_width, cos, sin, rot, q_norm, k_norm, eps, q_out, k_pages, v_pages, cache_dtype, tok_pos,
+                                 tok_seq, block_table, bt_stride, n_tokens, n_heads, n_kv_heads, dim, vdim, pad, stream));
+  RB_REQUIRE(n_tokens >= 0 && n_heads > 0 && n_kv_heads >= 0 && dim > 0 && vdim > 0 && pad >= dim && pad >= vdim,
+             "rb_norm_rope_store: bad sizes T=%d Hq=%d Hk=%d dim=%d vdim=%d pad=%d", n_tokens, n_heads, n_kv_heads, dim, vdim, pad);
+  RB_REQUIRE(rot >= 0 && rot % 2 == 0 && rot <= dim, "rb_norm_rope_store: %d rotated numbers in a head of %d", rot, dim);
+  RB_REQUIRE(rot == 0 || (cos != nullptr && sin != nullptr), "rb_norm_rope_store: a rotation needs its tables");
+  RB_REQUIRE(q_norm != nullptr && (k_pages == nullptr || k_norm != nullptr), "rb_norm_rope_store: the norms' weights are needed");
+  RB_REQUIRE((k_pages == nullptr) == (v_pages == nullptr), "rb_norm_rope_store: k and v pages go together");
+  const long long need = (long long)n_heads * dim + (k_pages ? (long long)n_kv_heads * (dim + vdim) : 0);
+  RB_REQUIRE(row_width >= need, "rb_norm_rope_store: rows of %lld numbers, %lld needed", row_width, need);
+  if (n_tokens == 0) return 0;
+  hipStream_t s = (hipStream_t)stream;
+  if (cache_dtype == RB_F32)
+    norm_rope_store_kernel<float><<<n_tokens, 256, 0, s>>>(qkv, (size_t)row_width, cos, sin, rot, q_norm, k_norm, eps, (float*)q_out,
+                                                           (float*)k_pages, (float*)v_pages, tok_pos, tok_seq, block_table,
+                                                           bt_stride, n_heads, n_kv_heads, dim, vdim, pad);
+  else if (cache_dtype == RB_BF16)
+    norm_rope_store_kernel<bf16_t><<<n_tokens, 256, 0, s>>>(qkv, (size_t)row_width, cos, sin, rot, q_norm, k_norm, eps,
+                                                            (bf16_t*)q_out, (bf16_t*)k_pages, (bf16_t*)v_pages, tok_pos, tok_seq,
+                                                            block_table, bt_stride, n_heads, n_kv_heads, dim, vdim, pad);
+  else
+    RB_REQUIRE(false, "rb_norm_rope_store: unknown dtype %d", cache_dtype);
+  RB_LAUNCH_CHECK();
+  return 0;
+}
+
+// ---------------------------------------------------------------- a gate on every number
+// x[e] *= sigmoid(gate[e]), in place; x of dtype and gate float32 laid out alike, n numbers.
+template <typename TC>
+__global__ void sigmoid_gate_kernel(TC* __restrict__ x, const float* __restrict__ gate, size_t n) {
+  for (size_t e = (size_t)blockIdx.x * blockDim.x + threadIdx.x; e < n; e += (size_t)gridDim.x * blockDim.x)
+    Num<TC>::store(x + e, Num<TC>::load(x + e) / (1.0f + expf(-gate[e])));
+}
+
+extern "C" int rb_sigmoid_gate(void* x, int dtype, const float* gate, long long n, void* stream) {
+  RB_RECORDED(rb_sigmoid_gate(x, dtype, gate, n, stream));
+  RB_REQUIRE(n >= 0, "rb_sigmoid_gate: bad size");
+  if (n == 0) return 0;
+  const size_t blocks = ((size_t)n + 255) / 256;
+  const int grid = (int)(blocks < 65535 ? blocks : 65535);
+  hipStream_t s = (hipStream_t)stream;
+  if (dtype == RB_F32)
+    sigmoid_gate_kernel<float><<<grid, 256, 0, s>>>((float*)x, gate, (size_t)n);
+  else if (dtype == RB_BF16)
+    sigmoid_gate_kernel<bf16_t><<<grid, 256, 0, s>>>((bf16_t*)x, gate, (size_t)n);
+  else
+    RB_REQUIRE(false, "rb_sigmoid_gate: unknown dtype %d", dtype);
+  RB_LAUNCH_CHECK();
+  return 0;
+}
+
+// ---------------------------------------------------------------- the token before, mixed in
+// out[m, t, :] = h[t] + (h[t - 1] - h[t]) * mu[m], m < n_mix, where the row before a step's first comes from the sequence's
+// state [slots, E] (float32; zeros for a fresh slot) and the state then holds the step's last row.  float32 arithmetic; h and
+// out of dtype.  A workgroup a token; the one that takes a sequence's first row of the step is also the one that writes
+// the state, after it has read it.
+template <typename TC>
+__global__ void shift_mix_kernel(const TC* __restrict__ h, float* __restrict__ state, const float* __restrict__ mu, int n_mix,
+                                 TC* __restrict__ out, const int32_t* __restrict__ cu_seqlens, const int32_t* __restrict__ tok_seq,
+                                 const int32_t* __restrict__ slots, int n_tokens, int width) {
+  const int t = blockIdx.x;
+  const int b = tok_seq[t];
+  const int row0 = cu_seqlens[b], last = cu_seqlens[b + 1] - 1;
+  const bool first = t == row0;
+  float* st = state + (size_t)slots[b] * width;
+  for (int j = threadIdx.x; j < width; j += blockDim.x) {
+    const float cur = Num<TC>::load(h + (size_t)t * width + j);
+    const float before = first ? st[j] : Num<TC>::load(h + (size_t)(t - 1) * width + j);
+    const float d = before - cur;
+    for (int m = 0; m < n_mix; ++m)
+      Num<TC>::store(out + ((size_t)m * n_tokens + t) * width + j, fmaf(d, mu[(size_t)m * width + j], cur));
+    if (first) st[j] = last == t ? cur : Num<TC>::load(h + (size_t)last * width + j);
+  }
+}
+
+extern "C" int rb_shift_mix(const void* h, int dtype, float* state, const float* mu, int n_mix, void* out,
+                            const int32_t* cu_seqlens, const int32_t* tok_seq, const int32_t* slots, int n_tokens, int n_seqs,
+                            int width, void* stream) {
+  RB_RECORDED(rb_shift_mix(h, dtype, state, mu, n_mix, out, cu_seqlens, tok_seq, slots, n_tokens, n_seqs, width, stream));
+  RB_REQUIRE(n_tokens >= 0 && n_seqs >= 0 && width > 0 && n_mix > 0, "rb_shift_mix: bad sizes");
+  RB_REQUIRE(h && state && mu && out, "rb_shift_mix: a pointer is missing");
+  if (n_tokens == 0) return 0;
+  hipStream_t s = (hipStream_t)stream;
+  const int threads = width >= 1024 ? 1024 : 256;
+  if (dtype == RB_F32)
+    shift_mix_kernel<float><<<n_tokens, threads, 0, s>>>((const float*)h, state, mu, n_mix, (float*)out, cu_seqlens, tok_seq, slots,
+                                                        n_tokens, width);
+  else if (dtype == RB_BF16)
+    shift_mix_kernel<bf16_t><<<n_tokens, threads, 0, s>>>((const bf16_t*)h, state, mu, n_mix, (bf16_t*)out, cu_seqlens, tok_seq,
+                                                         slots, n_tokens, width);
+  else
+    RB_REQUIRE(false, "rb_shift_mix: unknown dtype %d", dtype);
+  RB_LAUNCH_CHECK();
+  return 0;
+}

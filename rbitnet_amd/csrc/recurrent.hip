@@ -21,7 +21,8 @@ __device__ __forceinline__ float rb_softplus(float v) { return v > 20.0f ? v : l
 #define SC_MAX_TAPS 16
 #define SC_TILE 16             // rows of the step that a workgroup walks
 template <typename TO>
-__global__ void short_conv_kernel(const float* __restrict__ x, size_t x_stride, const float* __restrict__ w, int taps,
+__global__ void short_conv_kernel(const float* __restrict__ x, size_t x_stride, const float* __restrict__ bias,
+                                  const float* __restrict__ w, int taps,
                                   float* __restrict__ state, const int32_t* __restrict__ tok_pos,
                                   const int32_t* __restrict__ tok_seq, const int32_t* __restrict__ cu_seqlens,
                                   const int32_t* __restrict__ slots, TO* __restrict__ out, size_t out_stride,
@@ -41,6 +42,7 @@ __global__ void short_conv_kernel(const float* __restrict__ x, size_t x_stride, 
         wt[j] = j < keep ? w[(size_t)c * taps + j] : 0.f;
       }
       const float w_cur = w[(size_t)c * taps + keep];
+      const float bc = bias ? bias[c] : 0.f;
       bool have = false;
       for (int t = r0; t < r1; ++t) {
         if (t - cu_seqlens[tok_seq[t]] < keep) {             // the sequence's workgroup takes it
@@ -50,10 +52,10 @@ __global__ void short_conv_kernel(const float* __restrict__ x, size_t x_stride, 
         if (!have) {
 #pragma unroll
           for (int j = 0; j < SC_MAX_TAPS; ++j)
-            if (j < keep) win[j] = x[(size_t)(t - keep + j) * x_stride + c];
+            if (j < keep) win[j] = x[(size_t)(t - keep + j) * x_stride + c] + bc;
           have = true;
         }
-        const float cur = x[(size_t)t * x_stride + c];
+        const float cur = x[(size_t)t * x_stride + c] + bc;
         float acc = residual ? cur : 0.f;
         acc = fmaf(w_cur, cur, acc);
 #pragma unroll
@@ -81,11 +83,12 @@ __global__ void short_conv_kernel(const float* __restrict__ x, size_t x_stride, 
       wt[j] = j < keep ? w[(size_t)c * taps + j] : 0.f;
     }
     const float w_cur = w[(size_t)c * taps + keep];
-    float nxt = first > 0 ? x[(size_t)row0 * x_stride + c] : 0.f;
+    const float bc = bias ? bias[c] : 0.f;
+    float nxt = first > 0 ? x[(size_t)row0 * x_stride + c] + bc : 0.f;
     __builtin_amdgcn_sched_barrier(0);                       // state, weights and the first row: one trip to memory together
     for (int i = 0; i < first; ++i) {
       const float cur = nxt;
-      if (i + 1 < first) nxt = x[(size_t)(row0 + i + 1) * x_stride + c];
+      if (i + 1 < first) nxt = x[(size_t)(row0 + i + 1) * x_stride + c] + bc;
       float acc = residual ? cur : 0.f;
       acc = fmaf(w_cur, cur, acc);
 #pragma unroll
@@ -100,7 +103,7 @@ __global__ void short_conv_kernel(const float* __restrict__ x, size_t x_stride, 
     }
 #pragma unroll
     for (int j = 0; j < SC_MAX_TAPS; ++j)
-      if (j < keep) st[(size_t)j * channels + c] = n > keep ? x[(size_t)(row0 + n - keep + j) * x_stride + c] : win[j];
+      if (j < keep) st[(size_t)j * channels + c] = n > keep ? x[(size_t)(row0 + n - keep + j) * x_stride + c] + bc : win[j];
   }
 }
 
@@ -110,6 +113,18 @@ extern "C" int rb_short_conv(const float* x, long long x_stride, const float* w,
                              int act, int n_tokens, int n_seqs, int channels, void* stream) {
   RB_RECORDED(rb_short_conv(x, x_stride, w, taps, state, tok_pos, tok_seq, cu_seqlens, slots, out, out_stride, out_dtype,
                             residual, act, n_tokens, n_seqs, channels, stream));
+  return rb_short_conv_bias(x, x_stride, nullptr, w, taps, state, tok_pos, tok_seq, cu_seqlens, slots, out, out_stride, out_dtype,
+                            residual, act, n_tokens, n_seqs, channels, stream);
+}
+
+// The same on x + bias (bias float32 [C], null: none): the bias belongs to the inputs, so the state holds them with it and
+// rows before a sequence's start stay zero.
+extern "C" int rb_short_conv_bias(const float* x, long long x_stride, const float* bias, const float* w, int taps, float* state,
+                                  const int32_t* tok_pos, const int32_t* tok_seq, const int32_t* cu_seqlens,
+                                  const int32_t* slots, void* out, long long out_stride, int out_dtype, int residual,
+                                  int act, int n_tokens, int n_seqs, int channels, void* stream) {
+  RB_RECORDED(rb_short_conv_bias(x, x_stride, bias, w, taps, state, tok_pos, tok_seq, cu_seqlens, slots, out, out_stride, out_dtype,
+                                 residual, act, n_tokens, n_seqs, channels, stream));
   RB_REQUIRE(n_tokens >= 0 && n_seqs >= 0 && channels > 0 && taps >= 1 && taps - 1 <= SC_MAX_TAPS,
              "rb_short_conv: bad sizes T=%d B=%d C=%d taps=%d (at most %d)", n_tokens, n_seqs, channels, taps, SC_MAX_TAPS + 1);
   RB_REQUIRE(x_stride >= channels && out_stride >= channels, "rb_short_conv: a row stride is shorter than the channels");
@@ -120,10 +135,10 @@ extern "C" int rb_short_conv(const float* x, long long x_stride, const float* w,
   dim3 grid(n_tiles + (taps > 1 ? n_seqs : 0), (channels + 255) / 256 < 64 ? (channels + 255) / 256 : 64);
   hipStream_t s = (hipStream_t)stream;
   if (out_dtype == RB_F32)
-    short_conv_kernel<float><<<grid, 256, 0, s>>>(x, (size_t)x_stride, w, taps, state, tok_pos, tok_seq, cu_seqlens, slots,
+    short_conv_kernel<float><<<grid, 256, 0, s>>>(x, (size_t)x_stride, bias, w, taps, state, tok_pos, tok_seq, cu_seqlens, slots,
                                                   (float*)out, (size_t)out_stride, residual, act, channels, n_tokens, n_tiles);
   else if (out_dtype == RB_BF16)
-    short_conv_kernel<bf16_t><<<grid, 256, 0, s>>>(x, (size_t)x_stride, w, taps, state, tok_pos, tok_seq, cu_seqlens, slots,
+    short_conv_kernel<bf16_t><<<grid, 256, 0, s>>>(x, (size_t)x_stride, bias, w, taps, state, tok_pos, tok_seq, cu_seqlens, slots,
                                                    (bf16_t*)out, (size_t)out_stride, residual, act, channels, n_tokens, n_tiles);
   else
     RB_REQUIRE(false, "rb_short_conv: unknown dtype %d", out_dtype);
@@ -137,6 +152,7 @@ extern "C" int rb_short_conv(const float* x, long long x_stride, const float* w,
 // `a` become decays, a_cols being H (one per head) or H * dim (one per head and key channel), h = i / (a_cols / H):
 //   decay 0:  exp(-exp(a_log[h]) * softplus(a + bias[i]))
 //   decay 1:  sigmoid(a + bias[i]) ^ (1 / tau), computed as exp(-softplus(-(a + bias[i])) / tau)
+//   decay 2:  exp(-exp(a + bias[i]))
 // beta[t, h] = sigmoid(b[t, h]) where b_in is given.
 __global__ __launch_bounds__(1024) void recurrence_prep_kernel(float* __restrict__ qk, size_t qk_stride, int n_kv, int dim, int unit,
                                   float* __restrict__ a, size_t a_stride, int a_cols, int decay, const float* __restrict__ bias,
@@ -165,8 +181,10 @@ __global__ __launch_bounds__(1024) void recurrence_prep_kernel(float* __restrict
     const float z = ar[i] + (bias ? bias[i] : 0.f);
     if (decay == 0)
       ar[i] = expf(-expf(a_log[i / per_head]) * rb_softplus(z));
-    else
+    else if (decay == 1)
       ar[i] = expf(-rb_softplus(-z) / tau);
+    else
+      ar[i] = expf(-expf(z));
   }
   if (b_in)
     for (int h = threadIdx.x; h < n_heads; h += blockDim.x) beta[(size_t)t * n_heads + h] = rb_sigmoid(b_in[(size_t)t * b_stride + h]);
@@ -178,12 +196,13 @@ extern "C" int rb_recurrence_prep(float* qk, long long qk_stride, int n_kv_heads
                                   void* stream) {
   RB_RECORDED(rb_recurrence_prep(qk, qk_stride, n_kv_heads, dim, unit, q_scale, unit_eps, a, a_stride, a_cols, decay, bias, a_log,
                                  tau, n_heads, b_in, b_stride, beta, n_tokens, stream));
-  RB_REQUIRE(n_tokens >= 0 && n_kv_heads > 0 && n_heads > 0 && dim > 0, "rb_recurrence_prep: bad sizes");
+  RB_REQUIRE(n_tokens >= 0 && n_kv_heads >= 0 && n_heads > 0 && dim > 0, "rb_recurrence_prep: bad sizes");      // no q/k heads: the decays alone
   RB_REQUIRE(a_cols == n_heads || a_cols == n_heads * dim, "rb_recurrence_prep: %d decays a token for %d heads of %d", a_cols,
              n_heads, dim);
   RB_REQUIRE(qk_stride >= 2LL * n_kv_heads * dim && a_stride >= a_cols && (b_in == nullptr || b_stride >= n_heads),
              "rb_recurrence_prep: a row stride is too short");
-  RB_REQUIRE((decay == 0 && a_log != nullptr) || (decay == 1 && tau > 0.f), "rb_recurrence_prep: decay %d lacks its constants", decay);
+  RB_REQUIRE((decay == 0 && a_log != nullptr) || (decay == 1 && tau > 0.f) || decay == 2,
+             "rb_recurrence_prep: decay %d lacks its constants", decay);
   RB_REQUIRE(b_in == nullptr || beta != nullptr, "rb_recurrence_prep: beta has nowhere to go");
   if (n_tokens == 0) return 0;
   // a step of few tokens has few workgroups, and a token's heads are a chain of trips to memory for each wave: more waves then
@@ -226,12 +245,12 @@ __device__ __forceinline__ float lanes_sum(float v) {
   return v;
 }
 
-template <int DKL, int RG, int CH>
+template <int DKL, int RG, int CH, bool BONUS>
 __global__ __launch_bounds__(RB_WAVE) void delta_rule_kernel(
     const float* __restrict__ q, const float* __restrict__ k, size_t qk_stride, const float* __restrict__ v,
     size_t v_stride, const float* __restrict__ g, size_t g_stride, const float* __restrict__ beta, float* __restrict__ state,
     const int32_t* __restrict__ cu_seqlens, const int32_t* __restrict__ slots, float* __restrict__ out, int n_heads,
-    int n_kv, int dim, int vdim, int g_per_head) {
+    int n_kv, int dim, int vdim, int g_per_head, const float* __restrict__ bonus) {
   constexpr int COLS = RB_WAVE / RG;
   constexpr int DK = DKL * RG;               // rows held, >= dim; rows beyond dim stay zero
   constexpr int NQ = DK * CH / RB_WAVE;      // q (or k, or g) values of a chunk per lane
@@ -266,6 +285,14 @@ __global__ __launch_bounds__(RB_WAVE) void delta_rule_kernel(
       const int r = rg * DKL + i;
       s[i] = (on && r < dim) ? S[r] : 0.f;
     }
+  }
+  // BONUS: the read-out sees the state as it was before the token, and the token's own k v^T times a weight per key
+  // channel: o = S^T q + v sum_i bonus_i k_i q_i;  then S <- diag(g) S + k v^T
+  float ub[DKL];
+#pragma unroll
+  for (int i = 0; i < DKL; ++i) {
+    const int r = rg * DKL + i;
+    ub[i] = (BONUS && r < dim) ? bonus[(size_t)h * dim + r] : 0.f;
   }
   float rq[NQ], rk[NQ], rgt[NQ], rv[NV], rb = 0.f;
   auto fetch = [&](int t0) {
@@ -317,6 +344,15 @@ __global__ __launch_bounds__(RB_WAVE) void delta_rule_kernel(
       for (int i = 0; i < DKL; i += 2) {
         const float k0 = sk[tt][rg * DKL + i], q0 = sq[tt][rg * DKL + i];
         const float k1 = sk[tt][rg * DKL + i + 1], q1 = sq[tt][rg * DKL + i + 1];
+        if (BONUS) {
+          dq0 = fmaf(s[i], q0, dq0);
+          dq1 = fmaf(s[i + 1], q1, dq1);
+          kq0 = fmaf(ub[i] * k0, q0, kq0);
+          kq1 = fmaf(ub[i + 1] * k1, q1, kq1);
+          s[i] *= sg[tt][rg * DKL + i];
+          s[i + 1] *= sg[tt][rg * DKL + i + 1];
+          continue;
+        }
         s[i] *= sg[tt][rg * DKL + i];
         s[i + 1] *= sg[tt][rg * DKL + i + 1];
         kv0 = fmaf(s[i], k0, kv0);
@@ -326,10 +362,10 @@ __global__ __launch_bounds__(RB_WAVE) void delta_rule_kernel(
         kq0 = fmaf(k0, q0, kq0);
         kq1 = fmaf(k1, q1, kq1);
       }
-      const float kv = lanes_sum<RG>(kv0 + kv1);
+      const float kv = BONUS ? 0.f : lanes_sum<RG>(kv0 + kv1);
       const float dq = lanes_sum<RG>(dq0 + dq1);
       const float kq = lanes_sum<RG>(kq0 + kq1);
-      const float u = beta ? bt * (vv - kv) : vv;       // without beta: the plain rule, S <- diag(g) S + k v^T
+      const float u = (!BONUS && beta) ? bt * (vv - kv) : vv;       // without beta: the plain rule, S <- diag(g) S + k v^T
 #pragma unroll
       for (int i = 0; i < DKL; ++i) s[i] = fmaf(sk[tt][rg * DKL + i], u, s[i]);
       if (rg == 0) so[tt][lane / RG] = fmaf(u, kq, dq);
@@ -362,16 +398,16 @@ __global__ __launch_bounds__(RB_WAVE) void delta_rule_kernel(
   }
 }
 
-template <int DKL, int RG, int CH>
+template <int DKL, int RG, int CH, bool BONUS>
 static void launch_delta_rule(const float* q, const float* k, size_t qk_stride, const float* v, size_t v_stride,
                               const float* g, size_t g_stride, const float* beta, float* state, const int32_t* cu_seqlens,
                               const int32_t* slots, float* out, int n_seqs, int n_heads, int n_kv, int dim, int vdim,
-                              int g_per_head, hipStream_t s) {
+                              int g_per_head, const float* bonus, hipStream_t s) {
   constexpr int COLS = RB_WAVE / RG;
   static_assert((DKL * RG * CH) % RB_WAVE == 0 && CH <= RB_WAVE && DKL % 4 == 0, "a chunk's values are dealt evenly to the lanes");
   dim3 grid(n_seqs, n_heads, (vdim + COLS - 1) / COLS);
-  delta_rule_kernel<DKL, RG, CH><<<grid, RB_WAVE, 0, s>>>(q, k, qk_stride, v, v_stride, g, g_stride, beta, state, cu_seqlens,
-                                                          slots, out, n_heads, n_kv, dim, vdim, g_per_head);
+  delta_rule_kernel<DKL, RG, CH, BONUS><<<grid, RB_WAVE, 0, s>>>(q, k, qk_stride, v, v_stride, g, g_stride, beta, state, cu_seqlens,
+                                                                 slots, out, n_heads, n_kv, dim, vdim, g_per_head, bonus);
 }
 
 extern "C" int rb_delta_rule(const float* q, const float* k, long long qk_stride, const float* v, long long v_stride,
@@ -391,6 +427,20 @@ extern "C" int rb_linear_recurrence(const float* q, const float* k, long long qk
                                     int n_heads, int n_kv_heads, int dim, int vdim, void* stream) {
   RB_RECORDED(rb_linear_recurrence(q, k, qk_stride, v, v_stride, g, g_stride, g_per_head, beta, state, cu_seqlens, slots, out, n_seqs,
                                    n_tokens, n_heads, n_kv_heads, dim, vdim, stream));
+  return rb_linear_recurrence_bonus(q, k, qk_stride, v, v_stride, g, g_stride, g_per_head, beta, nullptr, state, cu_seqlens, slots,
+                                    out, n_seqs, n_tokens, n_heads, n_kv_heads, dim, vdim, stream);
+}
+
+// bonus (float32 [H, dim], null: rb_linear_recurrence): the plain rule read BEFORE the token's write, with the token's own
+// k v^T weighted per key channel:  out = (S + diag(bonus) k v^T)^T q;  S <- diag(g) S + k v^T.  Goes without beta.
+extern "C" int rb_linear_recurrence_bonus(const float* q, const float* k, long long qk_stride, const float* v, long long v_stride,
+                                          const float* g, long long g_stride, int g_per_head, const float* beta,
+                                          const float* bonus, float* state, const int32_t* cu_seqlens, const int32_t* slots,
+                                          float* out, int n_seqs, int n_tokens, int n_heads, int n_kv_heads, int dim, int vdim,
+                                          void* stream) {
+  RB_RECORDED(rb_linear_recurrence_bonus(q, k, qk_stride, v, v_stride, g, g_stride, g_per_head, beta, bonus, state, cu_seqlens, slots,
+                                         out, n_seqs, n_tokens, n_heads, n_kv_heads, dim, vdim, stream));
+  RB_REQUIRE(bonus == nullptr || beta == nullptr, "rb_linear_recurrence: a bonus goes with the plain rule (no beta)");
   RB_REQUIRE(n_seqs >= 0 && n_heads > 0 && n_kv_heads > 0 && n_heads % n_kv_heads == 0 && dim > 0 && vdim > 0,
              "rb_linear_recurrence: bad sizes H=%d Hk=%d dim=%d vdim=%d", n_heads, n_kv_heads, dim, vdim);
   RB_REQUIRE(g_stride >= (long long)n_heads * (g_per_head ? 1 : dim), "rb_linear_recurrence: the decays' row stride is too short");
@@ -405,12 +455,18 @@ extern "C" int rb_linear_recurrence(const float* q, const float* k, long long qk
 #define DR_GO(DKL, RG, CH)                                                                                                  \
   do {                                                                                                                      \
     constexpr int CH1 = (DKL * RG >= RB_WAVE) ? 1 : RB_WAVE / (DKL * RG);                                                   \
-    if (single)                                                                                                             \
-      launch_delta_rule<DKL, RG, CH1>(q, k, qs, v, vs, g, (size_t)g_stride, beta, state, cu_seqlens, slots, out, n_seqs,   \
-                                      n_heads, n_kv_heads, dim, vdim, g_per_head, s);                                       \
+    if (single && bonus)                                                                                                    \
+      launch_delta_rule<DKL, RG, CH1, true>(q, k, qs, v, vs, g, (size_t)g_stride, beta, state, cu_seqlens, slots, out,     \
+                                            n_seqs, n_heads, n_kv_heads, dim, vdim, g_per_head, bonus, s);                  \
+    else if (single)                                                                                                        \
+      launch_delta_rule<DKL, RG, CH1, false>(q, k, qs, v, vs, g, (size_t)g_stride, beta, state, cu_seqlens, slots, out,    \
+                                             n_seqs, n_heads, n_kv_heads, dim, vdim, g_per_head, bonus, s);                 \
+    else if (bonus)                                                                                                         \
+      launch_delta_rule<DKL, RG, CH, true>(q, k, qs, v, vs, g, (size_t)g_stride, beta, state, cu_seqlens, slots, out,      \
+                                           n_seqs, n_heads, n_kv_heads, dim, vdim, g_per_head, bonus, s);                   \
     else                                                                                                                    \
-      launch_delta_rule<DKL, RG, CH>(q, k, qs, v, vs, g, (size_t)g_stride, beta, state, cu_seqlens, slots, out, n_seqs,    \
-                                     n_heads, n_kv_heads, dim, vdim, g_per_head, s);                                        \
+      launch_delta_rule<DKL, RG, CH, false>(q, k, qs, v, vs, g, (size_t)g_stride, beta, state, cu_seqlens, slots, out,     \
+                                            n_seqs, n_heads, n_kv_heads, dim, vdim, g_per_head, bonus, s);                  \
   } while (0)
   // Rows of a column over RG lanes, chunks as long as the registers that hold the next one allow.  A token's time is
   // its lane's share of the column, so while the waves do not fill the GPU's SIMDs a column goes to more lanes
@@ -442,7 +498,7 @@ extern "C" int rb_linear_recurrence(const float* q, const float* k, long long qk
 template <typename TO>
 __global__ void gated_rmsnorm_kernel(const float* __restrict__ o, const float* __restrict__ weight,
                                      const float* __restrict__ gate, size_t gate_stride, float eps, TO* __restrict__ out,
-                                     int n_heads, int vdim, long long n_pairs, int act) {
+                                     int n_heads, int vdim, long long n_pairs, int act, size_t weight_head_stride) {
   const long long pair = (long long)blockIdx.x * (blockDim.x / RB_WAVE) + threadIdx.x / RB_WAVE;
   if (pair >= n_pairs) return;
   const int lane = threadIdx.x & (RB_WAVE - 1);
@@ -450,12 +506,13 @@ __global__ void gated_rmsnorm_kernel(const float* __restrict__ o, const float* _
   const int h = (int)(pair % n_heads);
   const float* p = o + (size_t)pair * vdim;
   const float* gp = gate + t * gate_stride + (size_t)h * vdim;
+  const float* wp = weight + (size_t)h * weight_head_stride;
   float ss = 0.f;
   for (int i = lane; i < vdim; i += RB_WAVE) ss = fmaf(p[i], p[i], ss);
   ss = wave_sum(ss);
   const float f = 1.0f / sqrtf(ss / (float)vdim + eps);
   for (int i = lane; i < vdim; i += RB_WAVE)
-    Num<TO>::store(out + (size_t)pair * vdim + i, p[i] * f * weight[i] * (act == 1 ? gp[i] * rb_sigmoid(gp[i]) : rb_sigmoid(gp[i])));
+    Num<TO>::store(out + (size_t)pair * vdim + i, p[i] * f * wp[i] * (act == 1 ? gp[i] * rb_sigmoid(gp[i]) : rb_sigmoid(gp[i])));
 }
 
 extern "C" int rb_gated_rmsnorm(const float* o, const float* weight, const float* gate, long long gate_stride, float eps,
@@ -468,6 +525,17 @@ extern "C" int rb_gated_rmsnorm(const float* o, const float* weight, const float
 extern "C" int rb_gated_rmsnorm_act(const float* o, const float* weight, const float* gate, long long gate_stride, int act, float eps,
                                     void* out, int out_dtype, int n_tokens, int n_heads, int vdim, void* stream) {
   RB_RECORDED(rb_gated_rmsnorm_act(o, weight, gate, gate_stride, act, eps, out, out_dtype, n_tokens, n_heads, vdim, stream));
+  return rb_gated_rmsnorm_heads(o, weight, 0, gate, gate_stride, act, eps, out, out_dtype, n_tokens, n_heads, vdim, stream);
+}
+
+// The same with head h's weight at weight + h * weight_head_stride (0: one weight of vdim numbers for all heads; vdim: a
+// weight over the concatenated heads).
+extern "C" int rb_gated_rmsnorm_heads(const float* o, const float* weight, long long weight_head_stride, const float* gate,
+                                      long long gate_stride, int act, float eps, void* out, int out_dtype, int n_tokens, int n_heads,
+                                      int vdim, void* stream) {
+  RB_RECORDED(rb_gated_rmsnorm_heads(o, weight, weight_head_stride, gate, gate_stride, act, eps, out, out_dtype, n_tokens, n_heads,
+                                     vdim, stream));
+  RB_REQUIRE(weight_head_stride >= 0, "rb_gated_rmsnorm: bad weight stride");
   RB_REQUIRE(n_tokens >= 0 && n_heads > 0 && vdim > 0 && (act == 0 || act == 1), "rb_gated_rmsnorm: bad sizes");
   RB_REQUIRE(gate_stride >= (long long)n_heads * vdim, "rb_gated_rmsnorm: the gate's row stride is too short");
   if (n_tokens == 0) return 0;
@@ -475,9 +543,11 @@ extern "C" int rb_gated_rmsnorm_act(const float* o, const float* weight, const f
   const int grid = (int)((n_pairs + 3) / 4);
   hipStream_t s = (hipStream_t)stream;
   if (out_dtype == RB_F32)
-    gated_rmsnorm_kernel<float><<<grid, 256, 0, s>>>(o, weight, gate, (size_t)gate_stride, eps, (float*)out, n_heads, vdim, n_pairs, act);
+    gated_rmsnorm_kernel<float><<<grid, 256, 0, s>>>(o, weight, gate, (size_t)gate_stride, eps, (float*)out, n_heads, vdim, n_pairs, act,
+                                                     (size_t)weight_head_stride);
   else if (out_dtype == RB_BF16)
-    gated_rmsnorm_kernel<bf16_t><<<grid, 256, 0, s>>>(o, weight, gate, (size_t)gate_stride, eps, (bf16_t*)out, n_heads, vdim, n_pairs, act);
+    gated_rmsnorm_kernel<bf16_t><<<grid, 256, 0, s>>>(o, weight, gate, (size_t)gate_stride, eps, (bf16_t*)out, n_heads, vdim, n_pairs, act,
+                                                      (size_t)weight_head_stride);
   else
     RB_REQUIRE(false, "rb_gated_rmsnorm: unknown dtype %d", out_dtype);
   RB_LAUNCH_CHECK();

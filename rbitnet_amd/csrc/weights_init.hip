@@ -164,6 +164,8 @@ extern "C" int rb_fill_normal(void* out, int dtype, long long n, unsigned long l
 extern "C" int rb_place_rows(const void* src, int src_dtype, void* dst, int dst_dtype, int dst_layout,
                              long long n_rows, long long width, long long dst_rows, long long row0, long long block,
                              long long period, void* stream) {
+  // also a step's cast of rows to the compute dtype, so it is noted like the kernels of a step
+  RB_RECORDED(rb_place_rows(src, src_dtype, dst, dst_dtype, dst_layout, n_rows, width, dst_rows, row0, block, period, stream));
   RB_REQUIRE(dst_layout == 0 || (dst_layout == 1 && dst_rows % 16 == 0 && width % (dst_dtype == RB_F32 ? 16 : 32) == 0),
              "rb_place_rows: layout %d of a destination of %lld rows of %lld", dst_layout, dst_rows, width);
   RB_REQUIRE(n_rows >= 0 && width > 0 && block > 0 && period >= block && row0 >= 0,

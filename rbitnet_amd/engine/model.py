@@ -194,7 +194,10 @@ class Model:
     def forward(self, ctx, cache, rows: torch.Tensor) -> torch.Tensor:
         """ctx.token_ids [T] -> float32 logits [len(rows), V] at the packed rows `rows`."""
         x = self.embedding.forward(ctx)
-        pending = run_blocks(self.blocks, self.spec.schedule, x, ctx, cache, getattr(self.head, "first_norm", None))
+        pending = None
+        if isinstance(x, tuple):              # an embedding may leave something for the first block (see stream.py)
+            x, pending = x
+        pending = run_blocks(self.blocks, self.spec.schedule, x, ctx, cache, getattr(self.head, "first_norm", None), pending)
         return self.head.forward(x, pending, rows, ctx)
 
 

@@ -28,6 +28,17 @@ and four more, each of which sends the layer through the kernels that take all h
   chunk       None, or c: a query at position i sees the keys j <= i with i // c == j // c only, chunks being counted
               from the sequence's first position, whatever a step brings.
 These go without a rotation (position "none") and without a sink.
+Five more send the layer through a third way, in which q, k and v are prepared by kernels of their own in front of attention
+(biases and a norm with a weight belong to it too, and a rotation is welcome):
+  conv        None, or the taps of a short causal convolution over time on every channel of q, k and v (tensors "q_conv",
+              "k_conv", "v_conv" [channels, taps], no bias), directly behind the projection and its bias; the last taps - 1
+              projected rows of a sequence are part of its state;
+  qk_norm     {"eps": e, "weight": True}: the norm of every query and key head has a weight of head_dim numbers that the heads
+              share (tensors "q_norm", "k_norm"), x / sqrt(mean(x^2) + e) * w, before the rotation;
+  softcap     None, or c: score <- c tanh(score / c) after the scale;
+  keep_first  with a window: the first keep_first tokens of a sequence stay visible behind it (at their own positions);
+  gate        "elementwise": the concatenated heads are multiplied number by number with sigmoid(Wg h) (tensor "gate"
+              [heads * value_dim, E]) before the output matrix.
 A position part that rotates only the first numbers of a head says so with its own head_dim
 (the table's width).  Where keys and values differ in size, or only a part of a head is
 rotated, queries, keys and values are laid out with one head size, the larger of the two,
@@ -54,9 +65,11 @@ import torch
 from ..errors import ConfigError
 from .base import BuildEnv, CacheRequest, Part, TensorSpec, build_part, register_mixer
 from .linear import linear, linear_or_terms, linear_to_stream, pack_rows
+from .short_conv import ACT_NONE, ShortConv
 
 DEFAULT_NAMES = {"q": "q_proj.weight", "k": "k_proj.weight", "v": "v_proj.weight", "o": "o_proj.weight", "sink": "sink",
-                 "gate": "gate", "q_bias": "q_proj.bias", "k_bias": "k_proj.bias", "v_bias": "v_proj.bias", "talk": "talk"}
+                 "gate": "gate", "q_bias": "q_proj.bias", "k_bias": "k_proj.bias", "v_bias": "v_proj.bias", "talk": "talk",
+                 "q_conv": "q.conv", "k_conv": "k.conv", "v_conv": "v.conv", "q_norm": "q.norm", "k_norm": "k.norm"}
 MIXED_MAX_HEADS, MIXED_MAX_NUMBERS = 64, 8192      # what the kernels that take all heads of a token together hold
 MIXED_MATRIX_CORE_HEADS = 32                       # and the one on the matrix cores
 _MATRIX_CORE_HEAD_DIMS = (64, 128)
@@ -106,8 +119,33 @@ class Attention(Part):
         self.chunk = None if params.get("chunk") is None else int(params["chunk"])
         if self.chunk is not None and self.chunk <= 0:
             raise ConfigError("attention: chunk must be positive")
+        # q, k and v prepared in front of attention: whenever one of these is asked for
+        self.taps = None if params.get("conv") is None else int(params["conv"])
+        self.qk_weight = bool(qk_norm and qk_norm.get("weight"))
+        self.softcap = None if params.get("softcap") is None else float(params["softcap"])
+        self.keep_first = int(params.get("keep_first") or 0)
+        self.gate_kind = str(params.get("gate") or ("head" if self.has_gate else "none"))
+        if self.gate_kind not in ("none", "head", "elementwise"):
+            raise ConfigError(f"attention: unknown gate {self.gate_kind!r} (head, elementwise)")
+        self.has_gate = self.gate_kind != "none"
+        if self.softcap is not None and not self.softcap > 0:
+            raise ConfigError("attention: softcap must be positive")
+        if self.keep_first < 0 or (self.keep_first and self.window is None):
+            raise ConfigError("attention: kept first tokens go with a window")
+        self.prepared = bool(self.taps is not None or self.qk_weight or self.softcap is not None or self.keep_first
+                             or self.gate_kind == "elementwise")
+        if self.prepared and (self.has_talk or self.chunk is not None):
+            raise ConfigError("attention: mixed heads and chunks go without a convolution, weighted norms, capped scores, "
+                              "kept first tokens and an elementwise gate")
+        self.conv = None
+        if self.prepared and (self.taps is not None or self.has_bias):
+            # a bias alone runs as a convolution of one tap (of ones): the same kernel adds it
+            n_ch = self.n_heads * self.head_dim
+            if self.cache_from is None:
+                n_ch += self.n_kv * (self.head_dim + self.value_dim)
+            self.conv = ShortConv(n_ch, self.taps or 1, env, residual=False, act=ACT_NONE)
         # all heads of a token in one workgroup: whenever one of the four is asked for
-        self.mixed = self.has_bias or self.has_talk or self.qk_eps is not None or self.chunk is not None
+        self.mixed = (not self.prepared) and (self.has_bias or self.has_talk or self.qk_eps is not None or self.chunk is not None)
         if self.mixed:
             if self.rot or self.has_sink:
                 raise ConfigError("attention: biases, unit heads, mixed heads and chunks go without a rotation and without a sink")
@@ -141,7 +179,18 @@ class Attention(Part):
         if self.has_sink:
             specs[self.names["sink"]] = TensorSpec((self.n_heads,), role="gain", init="normal")
         if self.has_gate:
-            specs[self.names["gate"]] = TensorSpec((self.n_heads, self.hidden))
+            rows = self.n_heads * (self.value_dim if self.gate_kind == "elementwise" else 1)
+            specs[self.names["gate"]] = TensorSpec((rows, self.hidden))
+        if self.taps is not None:
+            gain = lambda rows: TensorSpec((rows, self.taps), role="gain", init="normal")
+            specs[self.names["q_conv"]] = gain(qd)
+            if self.cache_from is None:
+                specs[self.names["k_conv"]] = gain(kd)
+                specs[self.names["v_conv"]] = gain(self.n_kv * self.value_dim)
+        if self.qk_weight:
+            specs[self.names["q_norm"]] = TensorSpec((self.head_dim,), role="gain", init="ones_normal")
+            if self.cache_from is None:
+                specs[self.names["k_norm"]] = TensorSpec((self.head_dim,), role="gain", init="ones_normal")
         return specs
 
     def load(self, tensors: Dict[str, torch.Tensor]) -> None:
@@ -173,27 +222,77 @@ class Attention(Part):
             self.talk = torch.eye(self.n_heads, dtype=torch.float32, device=o.device)
         if self.has_sink:
             self.sink = tensors[self.names["sink"]]
-        if self.has_gate:
+        if self.gate_kind == "head":
             # rows up to a multiple of 16 (zeros), so that the product's kernels find whole tiles
             g = tensors[self.names["gate"]]
             rows = (self.n_heads + 15) // 16 * 16
             full = torch.zeros((rows, self.hidden), dtype=g.dtype, device=g.device)
             full[:self.n_heads] = g
             self.w_gate = pack_rows(lib, [(full, 0, None, None)], rows, self.hidden, g.dtype, g.device, allowed)
+        elif self.gate_kind == "elementwise":
+            # the gate's rows in the layout of attention's output: heads of `pad` numbers, zero rows behind a head's values
+            g = tensors[self.names["gate"]]
+            full = torch.zeros((self.n_heads, self.pad, self.hidden), dtype=g.dtype, device=g.device)
+            full[:, :self.value_dim] = g.view(self.n_heads, self.value_dim, self.hidden)
+            self.w_gate = pack_rows(lib, [(full.view(-1, self.hidden), 0, None, None)], self.n_heads * self.pad, self.hidden,
+                                    g.dtype, g.device, allowed)
+        if self.conv is not None:
+            if self.taps is not None:
+                self.conv.load(torch.cat([tensors[self.names[n + "_conv"]] for n in names]))
+            else:
+                self.conv.load(torch.ones((self.conv.channels, 1), dtype=torch.float32, device=o.device))
+        if self.qk_weight:
+            self.q_norm_w = tensors[self.names["q_norm"]]
+            self.k_norm_w = tensors[self.names["k_norm"]] if self.cache_from is None else None
+        elif self.prepared and self.qk_eps is not None:
+            self.q_norm_w = self.k_norm_w = torch.ones(self.head_dim, dtype=torch.float32, device=o.device)
 
     def cache_request(self) -> Optional[CacheRequest]:
         if self.cache_from is not None:
             return None
         return CacheRequest("kv", heads=self.n_kv, head_dim=self.pad,
-                            window=None if self.window is None else int(self.window))
+                            window=None if self.window is None else int(self.window), keep_first=self.keep_first)
+
+    def cache_requests(self):
+        out = [r for r in (self.cache_request(),) if r is not None]
+        state = self.conv.cache_request("qkv_conv") if self.conv is not None else None
+        return out + ([state] if state is not None else [])
 
     # ------------------------------------------------------------------ forward
     def _gate_and_project(self, attn, h, stream, next_norm):
         lib = self.env.lib
-        if self.has_gate:
+        if self.gate_kind == "head":
             logits = linear(lib, h, self.w_gate, torch.float32)
             lib.head_gate(attn, logits, 0, self.n_heads, self.pad)
+        elif self.gate_kind == "elementwise":
+            lib.sigmoid_gate(attn, linear(lib, h, self.w_gate, torch.float32))
         return linear_to_stream(lib, attn, self.w_o, stream, next_norm)
+
+    def _forward_prepared(self, h, ctx, view, stream, next_norm):
+        """Bias and convolution, norms with weights, rotation and the cache write by kernels of their own; attention with
+        capped scores and kept first tokens; the gate."""
+        lib = self.env.lib
+        t, hq, hk, d = h.shape[0], self.n_heads, self.n_kv, self.pad
+        owns = self.cache_from is None
+        qkv = linear(lib, h, self.w_qkv, torch.float32)
+        if self.conv is not None:
+            qkv = self.conv.forward(qkv, ctx, view.states.get("qkv_conv"), torch.float32, bias=self.bias)
+        q = torch.empty((t, hq, d), dtype=self.env.dtype, device=h.device)
+        cos, sin, style = self.position.rotation_tables() if self.rot else (None, None, 1)
+        if self.rot and style != 1:
+            raise ConfigError("attention: a head prepared in front of attention pairs i with i + rot / 2 (style 'half')")
+        k_pages, v_pages = (view.k_pages, view.v_pages) if owns else (None, None)
+        if self.qk_eps is not None:
+            lib.norm_rope_store(qkv, cos, sin, self.rot, self.q_norm_w, self.k_norm_w, self.qk_eps, q, k_pages, v_pages,
+                                ctx.tok_pos, ctx.tok_seq, view.block_table, hq, hk, self.head_dim, self.value_dim, d)
+        else:
+            lib.rope_store(qkv, cos, sin, self.rot, q, k_pages, v_pages, ctx.tok_pos, ctx.tok_seq, view.block_table, hq, hk,
+                           self.head_dim, self.value_dim, d)
+        attn = torch.empty((t, hq * d), dtype=self.env.dtype, device=h.device)
+        window = int(self.window) if self.window is not None else 0
+        lib.attention_opts(q, view.k_pages, view.v_pages, attn, ctx.tok_pos, ctx.tok_seq, view.block_table, hq, hk, d,
+                           self.scale, window, self.keep_first, self.softcap or 0.0, self.sink)
+        return self._gate_and_project(attn, h, stream, next_norm)
 
     def _forward_mixed(self, h, ctx, view, stream, next_norm):
         """Biases, unit heads, the cache write, and attention with all heads of a token together."""
@@ -224,6 +323,10 @@ class Attention(Part):
         return self._gate_and_project(attn, h, stream, next_norm)
 
     def forward(self, h, ctx, view, stream: Optional[torch.Tensor] = None, next_norm=None):
+        if self.prepared:
+            if hasattr(h, "tensor") and not isinstance(h, torch.Tensor):
+                h = h.tensor()
+            return self._forward_prepared(h, ctx, view, stream, next_norm)
         if self.mixed:
             if hasattr(h, "tensor") and not isinstance(h, torch.Tensor):
                 h = h.tensor()

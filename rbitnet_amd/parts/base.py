@@ -35,7 +35,7 @@ class TensorSpec:
     role "gain":   a norm's gain, held in float32 (widening is exact);
     role "table":  integers, held as int32.
     init names the random initialisation: "normal" is N(0, std), "ones_normal"
-    is 1 + N(0, norm_std), "eye_normal" the identity matrix + N(0, norm_std)."""
+    is 1 + N(0, norm_std), "zero_normal" N(0, norm_std), "eye_normal" the identity matrix + N(0, norm_std)."""
     shape: Tuple[int, ...]
     role: str = "matrix"
     init: str = "normal"
@@ -61,7 +61,8 @@ class CacheRequest:
 
     kind "kv":    keys and values per token, `heads` x `head_dim` each; `window`
                   (None = all) is how far back a query looks, so that pages
-                  behind it can be given back.
+                  behind it can be given back; `keep_first` tokens at a sequence's
+                  start stay visible behind the window, and their pages are kept.
     kind "state": `state_shape` numbers per sequence, set to `state_init` when a
                   slot is handed out.
     Layers with equal requests share one group of storage.  A layer may ask for several things
@@ -77,10 +78,11 @@ class CacheRequest:
     state_dtype: torch.dtype = torch.float32
     name: str = ""
     values: bool = True
+    keep_first: int = 0
 
     def key(self) -> Tuple:
         return (self.kind, self.heads, self.head_dim, self.window, tuple(self.state_shape),
-                self.state_init, self.state_dtype, self.name, self.values)
+                self.state_init, self.state_dtype, self.name, self.values, self.keep_first)
 
 
 class Part:

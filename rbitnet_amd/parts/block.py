@@ -32,7 +32,7 @@ import torch
 from .base import BuildEnv, Part, TensorSpec, build_part, register_block
 from ..errors import ConfigError
 from .short_conv import ACT_NONE, ShortConv
-from .stream import GainedRows, ScaledSum, normed_for, sublayer  # noqa: F401  (normed_for: its old home)
+from .stream import GainedRows, ScaledSum, StreamCopy, WeightedTerms, normed_for, sublayer  # noqa: F401  (normed_for: its old home)
 
 DEFAULT_SEGMENTS = {"norm1": "input_layernorm", "mixer": "self_attn", "norm2": "post_attention_layernorm",
                     "feed_forward": "mlp"}
@@ -174,5 +174,85 @@ class ParallelBlock:
         return ScaledSum(a, b, self.scale)
 
 
+class OutNormBlock:
+    """"outnorm": the norms stand on the sublayers' outputs, and the sublayers read the stream itself:
+        x += norm1(mixer(x));  x += norm2(feed_forward(x))
+    The feed-forward (and norm2) may be left out.  The norms must offer `add_normed` (rmsnorm does): one kernel norms the
+    sublayer's output, adds it to the float32 stream and leaves the new rows in the compute dtype, which is what the next
+    sublayer, or the next such block, reads (`StreamCopy`).  A mixer that hands back `WeightedTerms` has them added up in
+    the same pass."""
+    takes_stream_copy = True
+    takes_next_norm = True
+
+    def __init__(self, layer_spec, env: BuildEnv):
+        self.env, self.hidden = env, env.hidden_size
+        self.norm1 = build_part("norm", layer_spec.norm1, env)
+        self.mixer = build_part("mixer", layer_spec.mixer, env)
+        self.norm2 = self.feed_forward = None
+        if layer_spec.feed_forward is not None:
+            self.norm2 = build_part("norm", layer_spec.norm2, env)
+            self.feed_forward = build_part("feed_forward", layer_spec.feed_forward, env)
+        self.segments = dict({"norm1": "norm1", "mixer": "mix", "norm2": "norm2", "feed_forward": "mlp"},
+                             **(getattr(layer_spec, "segments", None) or {}))
+        for norm in (self.norm1, self.norm2):
+            if norm is not None and not hasattr(norm, "add_normed"):
+                raise ConfigError("a layer with norms on its sublayers' outputs needs norms that can stand there (rmsnorm)")
+
+    def _all(self):
+        return [p for p in (self.norm1, self.mixer, self.norm2, self.feed_forward) if p is not None]
+
+    @property
+    def graph_safe(self) -> bool:
+        return all(getattr(p, "graph_safe", False) for p in self._all())
+
+    @property
+    def plan_safe(self) -> bool:
+        return all(getattr(p, "plan_safe", False) for p in self._all())
+
+    def parts(self) -> Dict[str, object]:
+        out = {self.segments["norm1"]: self.norm1, self.segments["mixer"]: self.mixer}
+        if self.feed_forward is not None:
+            out[self.segments["norm2"]] = self.norm2
+            out[self.segments["feed_forward"]] = self.feed_forward
+        return out
+
+    def cache_requests(self):
+        many = getattr(self.mixer, "cache_requests", None)
+        one = getattr(self.mixer, "cache_request", None)
+        return list(many()) if many else ([one()] if one and one() is not None else [])
+
+    def _rows(self, x: torch.Tensor) -> torch.Tensor:
+        return x if self.env.dtype == torch.float32 else torch.empty(x.shape, dtype=self.env.dtype, device=x.device)
+
+    def _add(self, norm, x: torch.Tensor, y) -> torch.Tensor:
+        """x += norm(y); returns the new rows in the compute dtype."""
+        h = self._rows(x)
+        out = None if h is x else h
+        if isinstance(y, WeightedTerms):
+            norm.add_normed(x, y.a, y.b, y.sa, y.sb, h_out=out)
+        else:
+            norm.add_normed(x, y, h_out=out)
+        return h
+
+    def forward(self, x: torch.Tensor, pending, ctx, view, next_norm=None):
+        if isinstance(pending, StreamCopy):
+            h = pending.h
+        else:
+            if pending is not None:
+                raise ConfigError("a layer with norms on its sublayers' outputs follows one that leaves the stream complete")
+            h = self._rows(x)
+            if h is not x:
+                self.env.lib.place_rows(x, h)
+        if getattr(self.mixer, "weighted_terms_ok", False):
+            y = self.mixer.forward(h, ctx, view, weighted_terms=True)
+        else:
+            y = self.mixer.forward(h, ctx, view)
+        h = self._add(self.norm1, x, y)
+        if self.feed_forward is not None:
+            h = self._add(self.norm2, x, self.feed_forward.forward(h, ctx))
+        return StreamCopy(h)
+
+
 register_block("prenorm", PreNormBlock)
+register_block("outnorm", OutNormBlock)
 register_block("parallel", ParallelBlock)

@@ -282,6 +282,78 @@ class DecayAttention(Part):
         return linear(lib, on, self.w_o, torch.float32)
 
 
+class TimeMix(Part):
+    """Time mixing with a token shift: a matrix state per head that decays per key channel, read BEFORE the token's own write,
+    with a bonus for the token itself.  With h' the row of the token before (zeros before a sequence's first):
+        m_s = h + (h' - h) * mu_s                                   for s in r, k, v, g, w: five inputs, one per projection
+        r, k, v = Wr m_r, Wk m_k, Wv m_v  (heads x dim each);  gate = silu(Wg m_g)
+        w = exp(-exp(Ww2 tanh(Ww1 m_w) + w0))                       per head and key channel, in float32
+        o = (S + diag(u) k v^T)^T r;   S <- diag(w) S + k v^T       u [heads, dim]: the bonus
+        o <- o / sqrt(mean(o^2) + eps) per head;  out = Wo (o * norm * gate)         norm [heads * dim]
+    The state S (`view.states["time_mix"]`, [slots, heads, dim, dim] float32, kept column by column) and the last row of h
+    (`view.states["time_shift"]`, float32) live in the cache's per-slot storage.  The recurrence is `rb_linear_recurrence`'s
+    kernel in its read-before-write form.
+    Parameters: heads, dim, decay_rank (the inner size of the decay's two matrices), eps, names."""
+    graph_safe = True
+    plan_safe = True
+
+    NAMES = {"mu_r": "mu.r", "mu_k": "mu.k", "mu_v": "mu.v", "mu_g": "mu.g", "mu_w": "mu.w", "r": "r", "k": "k", "v": "v", "g": "g",
+             "w1": "w1", "w2": "w2", "w0": "w0", "u": "u", "norm": "norm", "o": "o"}
+
+    def __init__(self, params: Dict, env: BuildEnv):
+        self.env = env
+        self.heads, self.dim = int(params["heads"]), int(params["dim"])
+        self.decay_rank = int(params["decay_rank"])
+        self.eps = float(params["eps"])
+        if min(self.heads, self.dim, self.decay_rank) <= 0 or self.dim > 512:
+            raise ConfigError("time mixing: sizes must be positive, the head size at most 512")
+        self.names = dict(self.NAMES, **(params.get("names") or {}))
+        self.hidden = env.hidden_size
+        self.n = self.heads * self.dim
+        self.cache_from = None
+
+    def tensor_specs(self) -> Dict[str, TensorSpec]:
+        n, e = self.names, self.hidden
+        gain = lambda *shape: TensorSpec(tuple(shape), role="gain", init="normal")
+        out = {n["mu_" + s]: gain(e) for s in "rkvgw"}
+        out.update({n[s]: TensorSpec((self.n, e)) for s in "rkvg"})
+        out.update({n["w1"]: TensorSpec((self.decay_rank, e)), n["w2"]: TensorSpec((self.n, self.decay_rank)), n["w0"]: gain(self.n),
+                    n["u"]: gain(self.heads, self.dim), n["norm"]: TensorSpec((self.n,), role="gain", init="ones_normal"),
+                    n["o"]: TensorSpec((e, self.n))})
+        return out
+
+    def load(self, tensors: Dict[str, torch.Tensor]) -> None:
+        lib, allowed, n = self.env.lib, not getattr(self.env, "generic_only", False), self.names
+        pack = lambda t: pack_rows(lib, [(t, 0, None, None)], t.shape[0], t.shape[1], t.dtype, t.device, allowed)
+        self.mu = torch.stack([tensors[n["mu_" + s]] for s in "rkvgw"]).contiguous()
+        self.w_in = [pack(tensors[n[s]]) for s in "rkvg"]
+        self.w_1, self.w_2, self.w_o = pack(tensors[n["w1"]]), pack(tensors[n["w2"]]), pack(tensors[n["o"]])
+        self.w0, self.u, self.norm = tensors[n["w0"]], tensors[n["u"]], tensors[n["norm"]]
+
+    def cache_requests(self) -> List[CacheRequest]:
+        return [CacheRequest("state", state_shape=(self.heads, self.dim, self.dim), state_init=0.0, name="time_mix"),
+                CacheRequest("state", state_shape=(self.hidden,), state_init=0.0, name="time_shift")]
+
+    def cache_request(self) -> Optional[CacheRequest]:
+        return self.cache_requests()[0]
+
+    def forward(self, h: torch.Tensor, ctx, view, stream: Optional[torch.Tensor] = None, next_norm=None) -> torch.Tensor:
+        lib, t, dt = self.env.lib, h.shape[0], self.env.dtype
+        mixes = torch.empty((5, t, self.hidden), dtype=dt, device=h.device)
+        lib.shift_mix(h, view.states["time_shift"], self.mu, ctx, mixes)
+        r, k, v, g = (linear(lib, mixes[i], self.w_in[i], torch.float32) for i in range(4))
+        low = torch.empty((t, self.decay_rank), dtype=dt, device=h.device)
+        lib.tanh_cast(linear(lib, mixes[4], self.w_1, torch.float32), low)
+        decay = linear(lib, low, self.w_2, torch.float32)
+        lib.decay_exp_exp(decay, self.w0, self.heads, self.dim)
+        o = torch.empty((t, self.n), dtype=torch.float32, device=h.device)
+        lib.time_mix_recurrence(r, k, v, decay, self.u, view.states["time_mix"], ctx, o, self.heads, self.dim, self.dim)
+        on = torch.empty((t, self.n), dtype=dt, device=h.device)
+        lib.gated_rmsnorm_heads(o, self.norm, g, 1, self.eps, self.heads, self.dim, on)
+        return linear(lib, on, self.w_o, torch.float32)
+
+
 register_mixer("channel_delta", ChannelDelta)
+register_mixer("time_mix", TimeMix)
 register_mixer("gated_delta", HeadDelta)
 register_mixer("decay_attention", DecayAttention)

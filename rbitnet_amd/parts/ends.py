@@ -10,7 +10,9 @@ embedding "table" (crates/bitnet-core/src/llama/model.rs:229-232): x[t, :] = tab
     Parameters: name, vocab_size, streams (None: the stream is [T, E]; n: n equal copies [n, T, E], for
     blocks that keep the residual stream in several copies), scale (None, or c: the rows are multiplied by c),
     positions (None, or {"name": tensor, "max_positions": n}: a learned vector per absolute position [n, E], added
-    to the scaled row as it is): x[t, :] = table[id[t], :] * c + positions[pos[t], :].
+    to the scaled row as it is): x[t, :] = table[id[t], :] * c + positions[pos[t], :]; norm (None, or a PartSpec of a norm
+    that offers `add_normed`) with norm_name (its tensor): the stream starts as norm(row), and the first block also gets
+    these rows in the compute dtype (forward then returns the stream and a `StreamCopy`).
     Interface of an embedding: tensor_specs() / load(tensors) / forward(ctx) -> float32 [T, E]
     (ctx.token_ids int32 [T]); `table` if a head may share it.
 
@@ -35,12 +37,10 @@ import torch
 from ..errors import ConfigError
 from .base import BuildEnv, Part, TensorSpec, build_part, register_embedding, register_head
 from .linear import linear, pack_rows
-from .stream import normed_for
+from .stream import StreamCopy, normed_for
 
 
 class TableEmbedding(Part):
-    graph_safe = True
-    plan_safe = True
 
     def __init__(self, params: Dict, env: BuildEnv):
         self.env = env
@@ -54,6 +54,12 @@ class TableEmbedding(Part):
         self.max_positions = None if pos is None else int(pos["max_positions"])
         if (self.scale is not None or pos is not None) and self.streams is not None:
             raise ConfigError("an embedding with a scale or learned positions fills one copy of the stream")
+        self.norm = None
+        if params.get("norm") is not None:
+            self.norm = build_part("norm", params["norm"], env)
+            self.norm_name = str(params["norm_name"])
+            if self.streams is not None or not hasattr(self.norm, "add_normed") or len(self.norm.tensor_specs()) != 1:
+                raise ConfigError("a norm behind the embedding: one copy of the stream, and a norm of one tensor that can stand on an output")
         self.table: Optional[torch.Tensor] = None
         self.positions: Optional[torch.Tensor] = None
 
@@ -61,12 +67,24 @@ class TableEmbedding(Part):
         out = {self.name: TensorSpec((self.vocab_size, self.hidden))}
         if self.pos_name is not None:
             out[self.pos_name] = TensorSpec((self.max_positions, self.hidden))
+        if self.norm is not None:
+            out[self.norm_name] = next(iter(self.norm.tensor_specs().values()))
         return out
 
     def load(self, tensors: Dict[str, torch.Tensor]) -> None:
         self.table = tensors[self.name]
         if self.pos_name is not None:
             self.positions = tensors[self.pos_name]
+        if self.norm is not None:
+            self.norm.load({next(iter(self.norm.tensor_specs())): tensors[self.norm_name]})
+
+    @property
+    def graph_safe(self) -> bool:
+        return self.norm is None or bool(getattr(self.norm, "graph_safe", False))
+
+    @property
+    def plan_safe(self) -> bool:
+        return self.norm is None or bool(getattr(self.norm, "plan_safe", False))
 
     def step_bytes(self, element_size: int) -> int:
         return 0                      # the gather reads a few rows only
@@ -82,6 +100,11 @@ class TableEmbedding(Part):
                                           self.positions, ctx.tok_pos, x)
         else:
             self.env.lib.embed_gather(self.table, ctx.token_ids, x)
+        if self.norm is not None:
+            rows = torch.empty((ctx.n_tokens, self.hidden), dtype=torch.float32, device=x.device)
+            h = rows if self.env.dtype == torch.float32 else torch.empty_like(rows, dtype=self.env.dtype)
+            self.norm.add_normed(rows, x, h_out=None if h is rows else h, assign=True)
+            return rows, StreamCopy(h)
         return x
 
 

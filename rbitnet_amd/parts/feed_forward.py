@@ -109,7 +109,44 @@ class DenseGelu(DenseAct):
     activation = "gelu_tanh"
 
 
+class ClampedGLU(Part):
+    """A gated feed-forward with limits on both branches:
+        g = min(Wgate h, limit),  u = clamp(Wup h, -limit, limit);  out = Wdown (g * sigmoid(alpha * g) * (u + 1))
+    (the unit of the routed experts, as a dense layer).  Gate and up are one product with float32 sums; limits, gate and
+    the rounding to the compute dtype are one kernel on them.
+    Parameters: intermediate_size, limit (None or <= 0: no limits), alpha (1.702), names ({"gate", "up", "down"})."""
+    graph_safe = True
+    plan_safe = True
+
+    def __init__(self, params: Dict, env: BuildEnv):
+        self.env = env
+        self.ff = int(params["intermediate_size"])
+        self.limit = float(params.get("limit") or 0.0)
+        self.alpha = float(params.get("alpha", 1.702))
+        self.names = dict({"gate": "gate", "up": "up", "down": "down"}, **(params.get("names") or {}))
+        self.hidden = env.hidden_size
+
+    def tensor_specs(self) -> Dict[str, TensorSpec]:
+        return {self.names["gate"]: TensorSpec((self.ff, self.hidden)), self.names["up"]: TensorSpec((self.ff, self.hidden)),
+                self.names["down"]: TensorSpec((self.hidden, self.ff))}
+
+    def load(self, tensors: Dict[str, torch.Tensor]) -> None:
+        allowed = not getattr(self.env, "generic_only", False)
+        self.w_gate_up = pack_gate_up(self.env.lib, tensors[self.names["gate"]], tensors[self.names["up"]], False, allowed)
+        down = tensors[self.names["down"]]
+        self.w_down = pack_rows(self.env.lib, [(down, 0, None, None)], down.shape[0], down.shape[1], down.dtype, down.device,
+                                allowed)
+
+    def forward(self, h, ctx=None, stream: Optional[torch.Tensor] = None, next_norm=None):
+        lib = self.env.lib
+        gu = linear(lib, h, self.w_gate_up, torch.float32)
+        t = torch.empty((h.shape[0], self.ff), dtype=self.env.dtype, device=gu.device)
+        lib.clamped_glu(gu, t, self.limit, self.alpha)
+        return linear(lib, t, self.w_down, torch.float32)
+
+
 register_feed_forward("swiglu", SwiGLU)
+register_feed_forward("clamped_glu", ClampedGLU)
 register_feed_forward("dense_xielu", DenseXielu)
 register_feed_forward("dense_gelu", DenseGelu)
 register_feed_forward("dense_act", DenseAct)

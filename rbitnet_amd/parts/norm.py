@@ -30,8 +30,12 @@ from .stream import GainedRows, ScaledSum, StreamsUpdate  # noqa: F401  (GainedR
 class RMSNorm(Part):
     """Parameters: size, eps, and two that a plain decoder leaves out: scalar (True: the gain is ONE number for all
     coordinates, a tensor without dimensions; it is spread over the width at load time, so that every kernel and every
-    folding of the norm into products serves as it is), names ({"weight": ...}: the tensor's name below the part's prefix;
-    an empty name is the prefix itself)."""
+    folding of the norm into products serves as it is), one_plus (True: the tensor holds the gain's distance from one, the
+    norm multiplies by 1 + w; the sum is done once, in float32, at load time), names ({"weight": ...}: the tensor's name
+    below the part's prefix; an empty name is the prefix itself).
+
+    `add_normed` is the norm on a sublayer's OUTPUT: x <- x + norm(sa a + sb b), for layers whose sublayers read the stream
+    itself; it also leaves the new rows in the compute dtype for the next sublayer."""
     graph_safe = True
     plan_safe = True
     folds_into_products = True
@@ -41,16 +45,25 @@ class RMSNorm(Part):
         self.size = int(params["size"])
         self.eps = float(params["eps"])
         self.scalar = bool(params.get("scalar", False))
+        self.one_plus = bool(params.get("one_plus", False))
         self.names = dict({"weight": "weight"}, **(params.get("names") or {}))
         self.env = env
         self.weight: Optional[torch.Tensor] = None
 
     def tensor_specs(self) -> Dict[str, TensorSpec]:
-        return {self.names["weight"]: TensorSpec(() if self.scalar else (self.size,), role="gain", init="ones_normal")}
+        init = "zero_normal" if self.one_plus else "ones_normal"
+        return {self.names["weight"]: TensorSpec(() if self.scalar else (self.size,), role="gain", init=init)}
 
     def load(self, tensors: Dict[str, torch.Tensor]) -> None:
         w = tensors[self.names["weight"]]
         self.weight = w.reshape(1).expand(self.size).contiguous() if self.scalar else w
+        if self.one_plus:
+            self.weight = (self.weight.to(torch.float32) + 1.0).contiguous()
+
+    def add_normed(self, x: torch.Tensor, a: torch.Tensor, b: Optional[torch.Tensor] = None, sa: float = 1.0, sb: float = 1.0,
+                   h_out: Optional[torch.Tensor] = None, assign: bool = False) -> None:
+        """x [T, E] float32 <- (assign ? 0 : x) + norm(sa a + sb b); h_out (compute dtype) gets the new rows."""
+        self.env.lib.outnorm_residual(x, a, b, sa, sb, self.weight, self.eps, assign, h_out)
 
     def forward(self, x: torch.Tensor, delta: Optional[torch.Tensor] = None,
                 rows: Optional[torch.Tensor] = None, out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:

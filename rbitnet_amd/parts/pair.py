@@ -8,7 +8,13 @@ the segments `left` and `right` below the pair's own prefix, the two norm weight
 of the cache: the pair hands on all their requests, which therefore need different names or kinds (one "kv" request
 and any number of named states can share a layer).
 
-Parameters: left, right (each {"kind", "params"}), eps, names ({"left_out", "right_out"}), segments ({"left", "right"}).
+With `combine = "weighted"` there are no norms and no weights of the pair's own: the result is
+    out = left_scale * a + right_scale * b
+which the pair hands, as `WeightedTerms`, to a block that asks for them (the norm on the sublayer's output adds them up in its
+own pass over the rows).
+
+Parameters: left, right (each {"kind", "params"}), eps, names ({"left_out", "right_out"}), segments ({"left", "right"}),
+combine ("norm_mean"; "weighted" with left_scale and right_scale).
 """
 from __future__ import annotations
 
@@ -18,6 +24,7 @@ import torch
 
 from ..errors import ConfigError
 from .base import BuildEnv, CacheRequest, Part, TensorSpec, _REGISTRIES, register_mixer
+from .stream import WeightedTerms
 
 DEFAULT_NAMES = {"left_out": "left.out", "right_out": "right.out"}
 DEFAULT_SEGMENTS = {"left": "left", "right": "right"}
@@ -34,7 +41,12 @@ def _build(spec, env: BuildEnv):
 class MixerPair(Part):
     def __init__(self, params: Dict, env: BuildEnv):
         self.env = env
-        self.eps = float(params["eps"])
+        self.combine = str(params.get("combine", "norm_mean"))
+        if self.combine not in ("norm_mean", "weighted"):
+            raise ConfigError(f"a pair of mixers: unknown way to combine {self.combine!r} (norm_mean, weighted)")
+        self.weighted_terms_ok = self.combine == "weighted"
+        self.eps = float(params.get("eps", 0.0))
+        self.scales = (float(params.get("left_scale", 1.0)), float(params.get("right_scale", 1.0)))
         self.names = dict(DEFAULT_NAMES, **(params.get("names") or {}))
         self.segments = dict(DEFAULT_SEGMENTS, **(params.get("segments") or {}))
         self.left, self.right = _build(params["left"], env), _build(params["right"], env)
@@ -61,14 +73,16 @@ class MixerPair(Part):
         for segment, part in self._sub():
             for name, ts in part.tensor_specs().items():
                 out[f"{segment}.{name}"] = ts
-        for key in ("left_out", "right_out"):
-            out[self.names[key]] = TensorSpec((self.hidden,), role="gain", init="ones_normal")
+        if self.combine == "norm_mean":
+            for key in ("left_out", "right_out"):
+                out[self.names[key]] = TensorSpec((self.hidden,), role="gain", init="ones_normal")
         return out
 
     def load(self, tensors: Dict[str, torch.Tensor]) -> None:
         for segment, part in self._sub():
             part.load({name: tensors[f"{segment}.{name}"] for name in part.tensor_specs()})
-        self.w_left, self.w_right = tensors[self.names["left_out"]], tensors[self.names["right_out"]]
+        if self.combine == "norm_mean":
+            self.w_left, self.w_right = tensors[self.names["left_out"]], tensors[self.names["right_out"]]
 
     def cache_requests(self) -> List[CacheRequest]:
         out: List[CacheRequest] = []
@@ -84,9 +98,14 @@ class MixerPair(Part):
         reqs = self.cache_requests()
         return reqs[0] if reqs else None
 
-    def forward(self, h: torch.Tensor, ctx, view, stream: Optional[torch.Tensor] = None, next_norm=None) -> torch.Tensor:
+    def forward(self, h: torch.Tensor, ctx, view, stream: Optional[torch.Tensor] = None, next_norm=None,
+                weighted_terms: bool = False):
         a = self.left.forward(h, ctx, view)
         b = self.right.forward(h, ctx, view)
+        if self.combine == "weighted":
+            if not weighted_terms:
+                raise ConfigError("a pair of mixers combined as a weighted sum needs a block that adds up its two terms (outnorm)")
+            return WeightedTerms(a, self.scales[0], b, self.scales[1])
         out = torch.empty((h.shape[0], self.hidden), dtype=torch.float32, device=h.device)
         self.env.lib.pair_norm_mean(a, self.w_left, b, self.w_right, self.eps, out)
         return out

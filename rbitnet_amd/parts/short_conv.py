@@ -41,10 +41,15 @@ class ShortConv:
     def load(self, weight: torch.Tensor) -> None:
         self.weight = weight.contiguous()
 
-    def forward(self, x: torch.Tensor, ctx, state: Optional[torch.Tensor], out_dtype: torch.dtype, col0: int = 0) -> torch.Tensor:
+    def forward(self, x: torch.Tensor, ctx, state: Optional[torch.Tensor], out_dtype: torch.dtype, col0: int = 0,
+                bias: Optional[torch.Tensor] = None) -> torch.Tensor:
         """x [T, W] float32; columns col0 .. col0 + channels go through the convolution -> [T, channels]; the
-        state then moves on by the step's rows."""
+        state then moves on by the step's rows.  bias (float32 [channels]): added to the inputs first; the state then holds
+        the inputs with it."""
         lib = self.env.lib
         out = torch.empty((x.shape[0], self.channels), dtype=out_dtype, device=x.device)
-        lib.short_conv(x, col0, self.channels, self.weight, state, ctx, out, self.residual, self.act)
+        if bias is not None:
+            lib.short_conv_bias(x, col0, self.channels, bias, self.weight, state, ctx, out, self.residual, self.act)
+        else:
+            lib.short_conv(x, col0, self.channels, self.weight, state, ctx, out, self.residual, self.act)
         return out

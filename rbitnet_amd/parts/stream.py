@@ -16,6 +16,12 @@ prepared for the norm that follows, `GainedRows`).  What a sublayer has not yet 
                     is still to be done; a norm that reads such a stream does it in its own pass over the rows
     ScaledSum       scale * (a + b) still to be added: the two sublayers of a layer whose mixer and feed-forward read
                     the same norm, and the layer's residual factor; a norm that says `adds_scaled_sum` takes it as delta
+    StreamCopy      nothing to add, and the stream's rows as they are in the compute dtype: what the sublayers of a layer
+                    whose norms stand on the sublayers' outputs read; only a block that says `takes_stream_copy` gets it
+                    (`run_blocks` drops it before any other block and before the head)
+
+A mixer may hand back `WeightedTerms` (sa * a + sb * b, not yet added up) to a block that asks for them: the norm on the
+sublayer's output then adds them up in its own pass.
 
 What a part or a norm can do, it says with class attributes; a part without any gets and
 returns plain tensors, a norm without any does every sum and every normalisation in its own
@@ -95,6 +101,20 @@ class ScaledSum:
         return self.a, self.b, self.scale
 
 
+class StreamCopy:
+    """The rows of the float32 stream x [T, E] in the compute dtype (x itself where that is float32)."""
+
+    def __init__(self, h: torch.Tensor):
+        self.h = h
+
+
+class WeightedTerms:
+    """sa * a + sb * b, two float32 terms [T, E] that whoever takes them adds up."""
+
+    def __init__(self, a: torch.Tensor, sa: float, b: torch.Tensor, sb: float):
+        self.a, self.sa, self.b, self.sb = a, float(sa), b, float(sb)
+
+
 def normed_for(part, norm, x: torch.Tensor, pending, rows: Optional[torch.Tensor] = None):
     """The input of `part`: the stream x, with `pending` added if that is a tensor, normalised
     by `norm` (all rows, or `rows`).  GainedRows that were made for this norm go on as they are
@@ -116,12 +136,13 @@ def sublayer(part, norm, x: torch.Tensor, pending, next_norm, *args):
     return part.forward(h, *args)
 
 
-def run_blocks(blocks: Sequence, schedule: Sequence[int], x: torch.Tensor, ctx, cache, last_norm=None):
+def run_blocks(blocks: Sequence, schedule: Sequence[int], x: torch.Tensor, ctx, cache, last_norm=None, pending=None):
     """The blocks in schedule order on the stream x; returns what the last one left pending.
-    last_norm: the norm that reads the stream after the last block."""
-    pending = None
+    last_norm: the norm that reads the stream after the last block; pending: what the embedding left."""
     for place, i in enumerate(schedule):
         block = blocks[i]
+        if isinstance(pending, StreamCopy) and not getattr(block, "takes_stream_copy", False):
+            pending = None
         view = cache.view(place, ctx.block_tables)
         if getattr(block, "takes_next_norm", False):
             after = blocks[schedule[place + 1]] if place + 1 < len(schedule) else None
@@ -129,7 +150,7 @@ def run_blocks(blocks: Sequence, schedule: Sequence[int], x: torch.Tensor, ctx, 
             pending = block.forward(x, pending, ctx, view, next_norm=next_norm)
         else:
             pending = block.forward(x, pending, ctx, view)
-    return pending
+    return None if isinstance(pending, StreamCopy) else pending
 
 
 def norm_adds_terms(norm) -> bool:

@@ -127,7 +127,7 @@ def random_tensor(name: str, spec: TensorSpec, seed: int, std: float, norm_std: 
     by the fill kernel, elsewhere by its host twin, with the same bits."""
     if spec.role == "table":
         raise ValueError(f"no random rule for integer table {name!r}")
-    mean, scale = (1.0, norm_std) if spec.init == "ones_normal" else (0.0, norm_std if spec.init == "eye_normal" else std)
+    mean, scale = (1.0, norm_std) if spec.init == "ones_normal" else (0.0, norm_std if spec.init in ("eye_normal", "zero_normal") else std)
     if spec.init == "eye_normal":         # a square matrix near the identity (a mixture of copies that keeps each)
         plain = TensorSpec(tuple(spec.shape), role=spec.role, init="normal")
         noise = random_tensor(name, plain, seed, norm_std, norm_std, torch.float32, device)
