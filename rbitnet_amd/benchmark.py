@@ -374,9 +374,38 @@ def pulunex_config(width: int, layers: int, heads: int, kv_heads: int, ff: int, 
             "logit_scale": 0.5, "norm": {"eps": 1e-5}, "layers": out}
 
 
+def menerax_config(width: int, layers: int, heads: int, kv_heads: int, ff: int, vocab: int, window: int = 1024, keep_first: int = 64,
+                   head: int = 128) -> dict:
+    """Groups of four layers with norms on the sublayers' outputs: three with attention through a latent (128 numbers a token
+    in the cache: a latent of 96 and a rotated part of 32) and one with windowed attention (kept first tokens, capped
+    scores, a convolution of four taps, heads of `head` numbers) beside time mixing with heads of 64; dense feed-forwards
+    with limits."""
+    latent = {"heads": heads, "dim": 64, "rot_dim": 32, "vdim": 64, "q_rank": max(256, width * 3 // 8), "kv_rank": 96, "scale": 96 ** -0.5,
+              "rot": {"base": 10000.0, "dims": 32}}
+    left = {"heads": heads * 64 // head, "kv_heads": max(1, kv_heads * 64 // head), "dim": head, "vdim": head, "conv": 4,
+            "rot": {"base": 500000.0, "dims": head // 2, "scaling": {"factor": 8.0, "low": 1.0, "high": 4.0, "original": 8192}},
+            "scale": head ** -0.5, "softcap": 30.0, "mask": {"size": window, "keep_first": keep_first}}
+    right = {"heads": max(1, width // 128), "dim": 64, "decay_rank": 64}
+    mlp = {"kind": "dense", "ff": ff, "limit": 7.0}
+    out = []
+    for i in range(layers):
+        if i % 4 == 2:
+            out.append({"type": "parallel", "mixer": {"left": dict(left), "right": dict(right), "left_scale": 0.6, "right_scale": 1.1},
+                        "mlp": dict(mlp)})
+        else:
+            out.append({"type": "latent_attention", "mixer": dict(latent), "mlp": dict(mlp)})
+    return {"architecture": "Menerax", "vocab": vocab, "width": width, "norm": {"eps": 1e-6}, "layers": out}
+
+
 # size -> (the design's configuration, then the shapes beside it: the Llama shape of equal width, depth and feed-forward
 # width, and for Pulunex the Tigutar model of those sizes too, whose routed experts and attention kernels are the like ones)
 DESIGN_SIZES = {
+    # Menerax beside the Tigutar model of those sizes (gated attention, windowed attention beside a linear recurrence) and the Llama shape
+    "menerax_w1024": (menerax_config(1024, 12, 16, 4, 4096, 32000), tigutar_config(1024, 12, 16, 4, 4096, 32000, experts=16),
+                      _other(1024, 4096, 16, 4, 64, 12, vocab=32000)),
+    "menerax_w2048": (menerax_config(2048, 16, 32, 8, 8192, 128256), tigutar_config(2048, 16, 32, 8, 8192, 128256, experts=16),
+                      _other(2048, 8192, 32, 8, 64, 16)),
+    "menerax_w4096": (menerax_config(4096, 8, 64, 16, 14336, 128256), dict(LLAMA3_8B, num_hidden_layers=8)),
     "pulunex_w1024": (pulunex_config(1024, 12, 16, 4, 4096, 32000), tigutar_config(1024, 12, 16, 4, 4096, 32000, experts=16),
                       _other(1024, 4096, 16, 4, 64, 12, vocab=32000)),
     "pulunex_w2048": (pulunex_config(2048, 16, 32, 8, 8192, 128256), tigutar_config(2048, 16, 32, 8, 8192, 128256, experts=16),
@@ -502,7 +531,7 @@ def main(argv=None) -> int:
                     help="no benchmark line: the named shape's decode products of 8 tokens beside a kernel that only "
                          "reads as many bytes")
     ap.add_argument("--design", default="", metavar="SIZE",
-                    help=f"no benchmark line: a Bagonex, Tigutar or Pulunex model of this size ({', '.join(sorted(DESIGN_SIZES))}) beside the Llama "
+                    help=f"no benchmark line: a Bagonex, Tigutar, Pulunex or Menerax model of this size ({', '.join(sorted(DESIGN_SIZES))}) beside the Llama "
                          "shape of equal width, depth and feed-forward width (Pulunex: beside Tigutar too): prefill and decode throughput, and the time per kernel")
     ap.add_argument("--tokens", default="1,8,64,512,2048", help="token counts of --planner-sweep")
     ap.add_argument("--sweep-detail", default=None, help="--planner-sweep: a file for every candidate's time")

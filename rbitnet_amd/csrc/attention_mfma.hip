@@ -29,7 +29,10 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void attn_prefill_kernel(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_pages, const bf16_t* __restrict__ v_pages,
     bf16_t* __restrict__ out, const int32_t* __restrict__ cu_seqlens, const int32_t* __restrict__ past_len,
     const int32_t* __restrict__ block_table, int bt_stride, int n_heads, int n_kv, float scale_log2, int window,
-    int gw, int paired, const float* __restrict__ sinks) {
+    int gw, int paired, const float* __restrict__ sinks, int keep_first, float cap, float cap_pre) {
+  // keep_first (with a window): the sequence's first keep_first keys stay visible behind the window; the tiles that hold
+  // them are walked first.  cap > 0: a raw score s becomes cap * tanh(s * cap_pre) (cap_pre = scale / cap) before the mask,
+  // and scale_log2 is then log2(e) alone.
   constexpr int KLD = D + 8;          // K tile row: D + 8 elements, rows 16 bytes apart in bank space
   constexpr int VLD = RB_PAGE + 8;    // V^T tile row: 64 keys + 8
   constexpr int DC = D / 8;           // 16-byte chunks per row
@@ -89,6 +92,9 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void attn_prefill_kernel(
   const int wg_lo = (window > 0 && wg_min_pos - window + 1 > 0) ? wg_min_pos - window + 1 : 0;
   const int first_tile = wg_lo / RB_PAGE;
   const int last_tile = (past + wg_q_end) / RB_PAGE;
+  const int kept_tiles = keep_first > 0 ? (keep_first + RB_PAGE - 1) / RB_PAGE : 0;
+  const int n_first = kept_tiles < first_tile ? kept_tiles : first_tile;      // tiles of kept keys in front of the window's
+  const int n_walk = n_first + last_tile - first_tile + 1;
   int wave_first = first_tile, wave_last = -1;
   int wave_min_pos = 0, wave_max_lo = 0;      // a tile all of whose keys lie in [wave_max_lo, wave_min_pos] needs no mask
   if (wave_on) {
@@ -130,7 +136,7 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void attn_prefill_kernel(
       for (int e = 0; e < 4; ++e) {
         const int key = kt * RB_PAGE + 4 * v_quad + e;
         // keys outside what the sequence holds may be anything, even NaN: make them zero
-        vreg[e] = (key <= kv_last && key >= wg_lo) ? load16(v_pages + base + (size_t)(4 * v_quad + e) * D + v_dchunk * 8)
+        vreg[e] = (key <= kv_last && (key >= wg_lo || key < keep_first)) ? load16(v_pages + base + (size_t)(4 * v_quad + e) * D + v_dchunk * 8)
                                                    : zero16();
       }
     }
@@ -173,16 +179,19 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void attn_prefill_kernel(
   // Tile kt is read from buffer (kt - first_tile) % 2 while tile kt + 1 comes from memory into
   // registers and, after the products, goes into the other buffer: one barrier a tile, behind
   // which everyone has finished reading what the tile after next will overwrite.
-  load_tile(first_tile);
+  auto tile_of = [&](int step) { return step < n_first ? step : first_tile + step - n_first; };
+  load_tile(tile_of(0));
   store_tile(0);
   __syncthreads();
-  for (int kt = first_tile; kt <= last_tile; ++kt) {
-    const int buf = (kt - first_tile) & 1;
+  for (int step = 0; step < n_walk; ++step) {
+    const int kt = tile_of(step);
+    const bool kept = kt < kept_tiles;           // a tile with kept keys: also for a wave whose window begins behind it, masked
+    const int buf = step & 1;
     const bf16_t* ks = ks2[buf];
     const bf16_t* vt = vt2[buf];
-    const bool next = kt + 1 <= last_tile;
-    if (next) load_tile(kt + 1);
-    if (wave_on && kt >= wave_first && kt <= wave_last) {
+    const bool next = step + 1 < n_walk;
+    if (next) load_tile(tile_of(step + 1));
+    if (wave_on && kt <= wave_last && (kept || kt >= wave_first)) {
 
     // ---- S^T = K Q^T: rows keys, columns queries.  The fragments of K come from LDS a few MFMAs
     // ahead of their use, one read behind every MFMA: left to itself the compiler asked for two
@@ -219,15 +228,24 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void attn_prefill_kernel(
     // ---- mask (only tiles that touch the diagonal or the window's edge), running maximum.
     // Scores stay unscaled: the scale is positive, so the maximum can be taken first and the
     // scale folded into the exponent's argument.
-    const bool edge = (kt * RB_PAGE + RB_PAGE - 1 > wave_min_pos) || (window > 0 && kt * RB_PAGE < wave_max_lo);
+    const bool edge = kept || (kt * RB_PAGE + RB_PAGE - 1 > wave_min_pos) || (window > 0 && kt * RB_PAGE < wave_max_lo);
     float mx = -INFINITY;
+    if (cap > 0.f) {
+      // cap * tanh(x) as cap - 2 cap / (2^(2 x log2 e) + 1), on the hardware's exponential and reciprocal
+      const float pre2 = 2.0f * LOG2E * cap_pre, cap2 = 2.0f * cap;
+#pragma unroll
+      for (int rt = 0; rt < 2; ++rt)
+#pragma unroll
+        for (int e = 0; e < 16; ++e)
+          sacc[rt][e] = fmaf(-cap2, __builtin_amdgcn_rcpf(__builtin_amdgcn_exp2f(sacc[rt][e] * pre2) + 1.0f), cap);
+    }
     if (edge) {
 #pragma unroll
       for (int rt = 0; rt < 2; ++rt)
 #pragma unroll
         for (int e = 0; e < 16; ++e) {
           const int key = kt * RB_PAGE + rt * 32 + 8 * (e / 4) + 4 * g + (e % 4);
-          if (key > qpos || key < q_lo) sacc[rt][e] = -INFINITY;
+          if (key > qpos || (key < q_lo && key >= keep_first)) sacc[rt][e] = -INFINITY;
         }
     }
 #pragma unroll
@@ -320,6 +338,22 @@ extern "C" int rb_attention_prefill_bf16_sinks(const void* q, const void* k_page
                                                const float* sinks, void* stream) {
   RB_RECORDED(rb_attention_prefill_bf16_sinks(q, k_pages, v_pages, out, cu_seqlens, past_len, block_table, bt_stride, n_seqs,
                                               max_q_len, n_heads, n_kv_heads, head_dim, scale, window, sinks, stream));
+  return rb_attention_prefill_bf16_opts(q, k_pages, v_pages, out, cu_seqlens, past_len, block_table, bt_stride, n_seqs, max_q_len,
+                                        n_heads, n_kv_heads, head_dim, scale, window, 0, 0.0f, sinks, stream);
+}
+
+// With kept first keys behind the window (j < keep_first stays visible) and capped scores (softcap > 0:
+// s <- softcap tanh(s / softcap) after the scale).
+extern "C" int rb_attention_prefill_bf16_opts(const void* q, const void* k_pages, const void* v_pages, void* out,
+                                              const int32_t* cu_seqlens, const int32_t* past_len,
+                                              const int32_t* block_table, int bt_stride, int n_seqs, int max_q_len,
+                                              int n_heads, int n_kv_heads, int head_dim, float scale, int window,
+                                              int keep_first, float softcap, const float* sinks, void* stream) {
+  RB_RECORDED(rb_attention_prefill_bf16_opts(q, k_pages, v_pages, out, cu_seqlens, past_len, block_table, bt_stride, n_seqs,
+                                             max_q_len, n_heads, n_kv_heads, head_dim, scale, window, keep_first, softcap, sinks,
+                                             stream));
+  RB_REQUIRE(keep_first >= 0 && softcap >= 0.f, "rb_attention_prefill_bf16: negative keep_first or softcap");
+  if (window == 0) keep_first = 0;
   RB_REQUIRE(n_seqs > 0 && max_q_len > 0, "rb_attention_prefill_bf16: empty batch");
   RB_REQUIRE(n_heads > 0 && n_kv_heads > 0 && n_heads % n_kv_heads == 0,
              "rb_attention_prefill_bf16: bad head counts Hq=%d Hk=%d", n_heads, n_kv_heads);
@@ -342,12 +376,13 @@ extern "C" int rb_attention_prefill_bf16_sinks(const void* q, const void* k_page
   const int paired = (nw == 4 && g_prefill_paired && (int)(grid.x * grid.y) > cus && (int)(grid.x * grid.y) <= 2 * cus) ? cus : 0;
   RB_REQUIRE(grid.y <= 65535 && grid.z <= 65535, "rb_attention_prefill_bf16: batch or head count too large");
   hipStream_t s = (hipStream_t)stream;
-  const float sl2 = scale * LOG2E;
+  const float sl2 = softcap > 0.f ? LOG2E : scale * LOG2E;
+  const float cap_pre = softcap > 0.f ? scale / softcap : 0.f;
 #define RB_PF(DV, NWV)                                                                                          \
   attn_prefill_kernel<DV, NWV><<<grid, 64 * NWV, 0, s>>>((const bf16_t*)q, (const bf16_t*)k_pages,              \
                                                          (const bf16_t*)v_pages, (bf16_t*)out, cu_seqlens,      \
                                                          past_len, block_table, bt_stride, n_heads, n_kv_heads, \
-                                                         sl2, window, gw, paired, sinks)
+                                                         sl2, window, gw, paired, sinks, keep_first, softcap, cap_pre)
   if (head_dim == 128) {
     if (nw == 8) RB_PF(128, 8);
     else RB_PF(128, 4);

@@ -184,6 +184,7 @@ class Kernels:
             "rb_outnorm_residual": [_P, _P, _P, _F, _F, _P, _F, _I, _P, _I, _I, _I, _P],
             "rb_clamped_glu": [_P, _P, _I, _I, _I, _F, _F, _P],
             "rb_tanh_cast": [_P, _P, _I, _L, _P],
+            "rb_attention_prefill_bf16_opts": [_P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _I, _I, _F, _P, _P],
             "rb_attention_generic_opts": [_P, _P, _P, _P, _I, _P, _P, _P, _I, _I, _I, _I, _I, _F, _I, _I, _F, _P, _P],
             "rb_norm_rope_store": [_P, _L, _P, _P, _I, _P, _P, _F, _P, _P, _P, _I, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _P],
             "rb_sigmoid_gate": [_P, _I, _P, _L, _P],
@@ -392,7 +393,8 @@ class Kernels:
                                                 int(window or 0), self._stream()))
 
     def attention_prefill_bf16(self, q, k_pages, v_pages, out, cu_seqlens, past_len, block_table, n_seqs,
-                               max_q_len, n_heads, n_kv, head_dim, scale, window, sinks=None) -> None:
+                               max_q_len, n_heads, n_kv, head_dim, scale, window, sinks=None, keep_first: int = 0,
+                               softcap: float = 0.0) -> None:
         n = q.shape[0]
         _check(q, "q", torch.bfloat16, (n, n_heads, head_dim))
         _check(k_pages, "k_pages", torch.bfloat16)
@@ -405,11 +407,11 @@ class Kernels:
         _check(block_table, "block_table", torch.int32)
         if sinks is not None:
             _check(sinks, "sinks", torch.float32, (n_heads,))
-        self._ok(self._lib.rb_attention_prefill_bf16_sinks(_ptr(q), _ptr(k_pages), _ptr(v_pages), _ptr(out),
-                                                           _ptr(cu_seqlens), _ptr(past_len), _ptr(block_table),
-                                                           block_table.shape[1], n_seqs, int(max_q_len), n_heads, n_kv,
-                                                           head_dim, float(scale), int(window or 0), _ptr(sinks),
-                                                           self._stream()))
+        self._ok(self._lib.rb_attention_prefill_bf16_opts(_ptr(q), _ptr(k_pages), _ptr(v_pages), _ptr(out),
+                                                          _ptr(cu_seqlens), _ptr(past_len), _ptr(block_table),
+                                                          block_table.shape[1], n_seqs, int(max_q_len), n_heads, n_kv,
+                                                          head_dim, float(scale), int(window or 0), int(keep_first or 0),
+                                                          float(softcap or 0.0), _ptr(sinks), self._stream()))
 
     def attention_decode_bf16(self, q, k_pages, v_pages, out, tok_pos, block_table, n_heads, n_kv, head_dim,
                               scale, window, n_splits, workspace, sinks=None) -> None:

@@ -197,7 +197,8 @@ class Model:
         pending = None
         if isinstance(x, tuple):              # an embedding may leave something for the first block (see stream.py)
             x, pending = x
-        pending = run_blocks(self.blocks, self.spec.schedule, x, ctx, cache, getattr(self.head, "first_norm", None), pending)
+        more = {} if pending is None else {"pending": pending}
+        pending = run_blocks(self.blocks, self.spec.schedule, x, ctx, cache, getattr(self.head, "first_norm", None), **more)
         return self.head.forward(x, pending, rows, ctx)
 
 

@@ -290,8 +290,14 @@ class Attention(Part):
                            self.head_dim, self.value_dim, d)
         attn = torch.empty((t, hq * d), dtype=self.env.dtype, device=h.device)
         window = int(self.window) if self.window is not None else 0
-        lib.attention_opts(q, view.k_pages, view.v_pages, attn, ctx.tok_pos, ctx.tok_seq, view.block_table, hq, hk, d,
-                           self.scale, window, self.keep_first, self.softcap or 0.0, self.sink)
+        fast = (self.env.dtype == torch.bfloat16 and d in _MATRIX_CORE_HEAD_DIMS and not getattr(self.env, "generic_only", False))
+        if fast and ctx.max_q_len > 1:
+            lib.attention_prefill_bf16(q, view.k_pages, view.v_pages, attn, ctx.cu_seqlens, ctx.past_len, view.block_table,
+                                       ctx.n_seqs, ctx.max_q_len, hq, hk, d, self.scale, window, sinks=self.sink,
+                                       keep_first=self.keep_first, softcap=self.softcap or 0.0)
+        else:
+            lib.attention_opts(q, view.k_pages, view.v_pages, attn, ctx.tok_pos, ctx.tok_seq, view.block_table, hq, hk, d,
+                               self.scale, window, self.keep_first, self.softcap or 0.0, self.sink)
         return self._gate_and_project(attn, h, stream, next_norm)
 
     def _forward_mixed(self, h, ctx, view, stream, next_norm):

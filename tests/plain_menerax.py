@@ -233,3 +233,66 @@ class PlainMenerax:
     def logits(self, tokens: List[int]) -> torch.Tensor:
         x = self.streams(tokens)[-1]
         return norm_around_zero(x, self.w["final.norm"], self.eps) @ self.w["head"].T
+
+
+# ---------------------------------------------------------------- random models for the tests
+def tensor_shapes(cfg: Dict) -> Dict[str, tuple]:
+    """Name -> shape of every tensor of a model; a parallel layer's `right` names its `decay_rank` here."""
+    e, v = cfg["width"], cfg["vocab"]
+    out = {"embed": (v, e), "embed.norm": (e,), "final.norm": (e,), "head": (v, e)}
+    for i, layer in enumerate(cfg["layers"]):
+        if layer.get("weights_of") is not None:
+            continue
+        p = f"l{i}."
+        out[p + "norm1"] = (e,)
+        m = layer["mixer"]
+        if layer["type"] == "latent_attention":
+            h, d, r, dv = m["heads"], m["dim"], m["rot_dim"], m["vdim"]
+            out.update({p + "mix.dq": (m["q_rank"], e), p + "mix.dq.norm": (m["q_rank"],), p + "mix.uq": (h * (d + r), m["q_rank"]),
+                        p + "mix.dkv": (m["kv_rank"] + r, e), p + "mix.dkv.norm": (m["kv_rank"],),
+                        p + "mix.uk": (h * d, m["kv_rank"]), p + "mix.uv": (h * dv, m["kv_rank"]), p + "mix.g": (h, e),
+                        p + "mix.o": (e, h * dv)})
+        else:
+            a, b = m["left"], m["right"]
+            q, k, val = a["heads"] * a["dim"], a["kv_heads"] * a["dim"], a["kv_heads"] * a["vdim"]
+            lp, rp = p + "mix.left.", p + "mix.right."
+            for name, rows in (("q", q), ("k", k), ("v", val)):
+                out.update({lp + name: (rows, e), lp + name + ".b": (rows,), lp + name + ".conv": (rows, a["conv"])})
+            out.update({lp + "q.norm": (a["dim"],), lp + "k.norm": (a["dim"],), lp + "g": (a["heads"] * a["vdim"], e),
+                        lp + "o": (e, a["heads"] * a["vdim"])})
+            n = b["heads"] * b["dim"]
+            out.update({rp + "mu." + s: (e,) for s in "rkvgw"})
+            out.update({rp + s: (n, e) for s in "rkvg"})
+            out.update({rp + "w1": (b["decay_rank"], e), rp + "w2": (n, b["decay_rank"]), rp + "w0": (n,),
+                        rp + "u": (b["heads"], b["dim"]), rp + "norm": (n,), rp + "o": (e, n)})
+        if layer.get("mlp") is not None:
+            ff = layer["mlp"]["ff"]
+            out.update({p + "norm2": (e,), p + "mlp.gate": (ff, e), p + "mlp.up": (ff, e), p + "mlp.down": (e, ff)})
+    return out
+
+
+def random_menerax_tensors(cfg: Dict, seed: int) -> Dict[str, torch.Tensor]:
+    """Weights that bfloat16 holds exactly, so that the oracle and a model loaded from a bfloat16 file see the same numbers.
+    Sizes are chosen so that every mechanism matters at tiny widths."""
+    g = torch.Generator().manual_seed(seed)
+    out = {}
+    for name, shape in tensor_shapes(cfg).items():
+        last = name.rsplit(".", 1)[-1]
+        if name.endswith("norm1") or name.endswith("norm2") or name in ("embed.norm", "final.norm"):
+            t = 0.2 * torch.randn(shape, generator=g)                      # stored around zero
+        elif name.endswith(".norm"):
+            t = 1.0 + 0.2 * torch.randn(shape, generator=g)                # plain weights
+        elif last == "conv":
+            t = 0.6 * torch.randn(shape, generator=g)
+        elif ".mu." in name:
+            t = torch.rand(shape, generator=g)
+        elif last == "w0":
+            t = -1.0 + 1.5 * torch.randn(shape, generator=g)               # decays from nearly 1 to nearly 0
+        elif last in ("u", "b"):
+            t = 0.5 * torch.randn(shape, generator=g)
+        elif name == "embed":
+            t = torch.randn(shape, generator=g)
+        else:
+            t = torch.randn(shape, generator=g) * (1.5 / math.sqrt(shape[-1]))
+        out[name] = t.to(torch.bfloat16).to(F64)
+    return out
