@@ -55,6 +55,8 @@ int rb_gemm_generic(const void* a, const void* w, int w_layout, void* c, int dty
 //               (16 gate rows, then the 16 up rows of the same columns); the result is
 //               silu(gate) * up, [M, N/2]
 // K must be a multiple of 8 (rows 16-byte aligned).
+// rb_gemm_bf16_act with epilogue 1 and act = two numbers (limit, alpha), limit > 0: the gated pair with limits,
+// g = min(gate, limit), u = clamp(up, -limit, limit), result g * sigmoid(alpha g) * (u + 1).
 // w_layout says how W is stored.  0: N rows of K values.  1: fragment-major (K % 64 == 0 and
 // N % 16 == 0 only): blocks of 16 rows x 32 depth values, 1 KB each, in the order [N / 16][K / 32];
 // inside a block, the value of row r and depth d lies at 8 * (16 * (d / 8) + r) + d % 8.  A wave

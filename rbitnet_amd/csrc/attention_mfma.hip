@@ -719,7 +719,9 @@ __global__ __launch_bounds__(64 * NW) void attn_decode_mfma_kernel(
     const float* __restrict__ sin_t, int style, bf16_t* k_pages, bf16_t* v_pages, bf16_t* __restrict__ out,
     const int32_t* __restrict__ tok_pos, const int32_t* __restrict__ block_table, int bt_stride, int n_heads,
     int n_kv, float scale_log2, int window, int n_splits, float* __restrict__ ws, int qkv_terms, size_t qkv_stride,
-    const float* __restrict__ sinks) {
+    const float* __restrict__ sinks, int keep_first, float cap, float cap_pre) {
+  // keep_first (with a window): the first keep_first keys stay visible behind the window; their pages are walked before the
+  // window's.  cap > 0: a raw score s becomes cap * tanh(s * cap_pre) (cap_pre = scale / cap), and scale_log2 is log2(e).
   constexpr int KS = D / 32;          // depth steps of the score product
   constexpr int DT = D / 16;          // d tiles of the output product
   constexpr int HALF = D / 2;
@@ -746,6 +748,11 @@ __global__ __launch_bounds__(64 * NW) void attn_decode_mfma_kernel(
   const int lo = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
   const int first_page = lo / RB_PAGE, last_page = pos / RB_PAGE;
   const int32_t* pages = block_table + (size_t)b * bt_stride;
+  // the pages are walked by a running number: those of kept keys that lie before the window's first page, then the window's
+  const int kept_pages = keep_first > 0 ? (keep_first + RB_PAGE - 1) / RB_PAGE : 0;
+  const int n_first = kept_pages < first_page ? kept_pages : first_page;
+  const int n_walk = n_first + last_page - first_page + 1;
+  auto page_of = [&](int w) { return w < n_first ? w : first_page + w - n_first; };
 
   // ---- A page's way from memory (its number in the table, then its rows) is the longest wait
   // of a short step, so it starts early: the numbers of the wave's first two pages are asked
@@ -754,9 +761,9 @@ __global__ __launch_bounds__(64 * NW) void attn_decode_mfma_kernel(
   // page before that.
   Frag8 kf[4][KS], kf_next[4][KS];
   const int pg_step = NW * n_splits;
-  const int pg_first = first_page + split + n_splits * wave;
-  int id_next = pg_first <= last_page ? pages[pg_first] : 0;                       // the page worked on next
-  int id_after = pg_first + pg_step <= last_page ? pages[pg_first + pg_step] : 0;  // the one after it
+  const int w_first = split + n_splits * wave;
+  int id_next = w_first < n_walk ? pages[page_of(w_first)] : 0;                       // the page worked on next
+  int id_after = w_first + pg_step < n_walk ? pages[page_of(w_first + pg_step)] : 0;  // the one after it
   uint16_t* vpage = vpages + wave * RB_PAGE * D;
   const uint32_t vpage_lds = (uint32_t)(uintptr_t)vpage;
   // ONCE >= 1: the pages of V, whole rows that are read once in a step, go past the caches; ONCE = 2: the
@@ -819,13 +826,13 @@ __global__ __launch_bounds__(64 * NW) void attn_decode_mfma_kernel(
     }
   }
   int page_cur = 0;
-  if (pg_first <= last_page) {
+  if (w_first < n_walk) {
     page_cur = __builtin_amdgcn_readfirstlane(id_next);
     ask_values(page_cur);
     ask_keys(page_cur);
   }
   __syncthreads();
-  if (FUSED && split == (last_page - first_page) % n_splits) {      // this workgroup owns the last page
+  if (FUSED && split == (n_walk - 1) % n_splits) {      // this workgroup owns the last page
     const int page = pages[last_page];
     const size_t at = ((size_t)page * n_kv + kvh) * RB_PAGE * D + (size_t)(pos % RB_PAGE) * D;
     for (int d = tid; d < D; d += NT) {
@@ -842,7 +849,8 @@ __global__ __launch_bounds__(64 * NW) void attn_decode_mfma_kernel(
 #pragma unroll
   for (int dt = 0; dt < DT; ++dt) acc_o[dt] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
 
-  for (int pg = pg_first; pg <= last_page; pg += pg_step) {
+  for (int w = w_first; w < n_walk; w += pg_step) {
+    const int pg = page_of(w);
     // This page's keys must all have arrived here, before the loads into LDS below are issued:
     // the compiler does not see those (they are assembly) and would count them out wrongly if
     // it waited for keys later.  Touching every register makes it wait now.
@@ -853,20 +861,20 @@ __global__ __launch_bounds__(64 * NW) void attn_decode_mfma_kernel(
         kf[t][st] = kf_next[t][st];
         asm volatile("" ::"v"(kf[t][st].u.x), "v"(kf[t][st].u.y), "v"(kf[t][st].u.z), "v"(kf[t][st].u.w) : "memory");
       }
-    if (pg != pg_first) {
+    if (w != w_first) {
       // the reads of the previous page have all returned before its area is overwritten (the
       // first page's values were asked for before the barrier)
       asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
       ask_values(page_cur);
     }
     // the next page's keys (its number was asked for a page ago), and the number of the one after
-    const bool more = pg + pg_step <= last_page;
-    const bool more2 = pg + 2 * pg_step <= last_page;
+    const bool more = w + pg_step < n_walk;
+    const bool more2 = w + 2 * pg_step < n_walk;
     int page_nx = 0;
     if (more) {
       page_nx = __builtin_amdgcn_readfirstlane(id_after);
       ask_keys(page_nx);
-      if (more2) id_after = pages[pg + 2 * pg_step];
+      if (more2) id_after = pages[page_of(w + 2 * pg_step)];
     }
     if (FUSED && pg == last_page) {
       // the token's own key is not in the cache yet (or only just): take it from LDS
@@ -891,7 +899,10 @@ __global__ __launch_bounds__(64 * NW) void attn_decode_mfma_kernel(
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         const int key = pg * RB_PAGE + 16 * t + 4 * grp + i;
-        const float v = (key >= lo && key <= pos) ? sc[t][i] * scale_log2 : -INFINITY;
+        float raw = sc[t][i];
+        if (cap > 0.f)      // cap * tanh(x) as cap - 2 cap / (2^(2 x log2 e) + 1)
+          raw = fmaf(-2.0f * cap, __builtin_amdgcn_rcpf(__builtin_amdgcn_exp2f(raw * (2.0f * LOG2E * cap_pre)) + 1.0f), cap);
+        const float v = (key <= pos && (key >= lo || key < keep_first)) ? raw * scale_log2 : -INFINITY;
         sc[t][i] = v;
         mx = fmaxf(mx, v);
       }
@@ -1046,6 +1057,9 @@ struct DecodeArgs {
   int qkv_terms;          // fused: qkv as so many terms to be added up, qkv_stride floats apart
   size_t qkv_stride;
   const float* sinks;     // per query head, or null
+  int keep_first = 0;     // with a window: the first keys that stay visible behind it
+  float cap = 0.f;        // > 0: scores capped at cap * tanh(score / cap); sl2 is then log2(e) and cap_pre scale / cap
+  float cap_pre = 0.f;
 };
 
 template <int D, int G, bool FUSED>
@@ -1071,7 +1085,7 @@ static int launch_decode_mfma_nw(const DecodeArgs& a, hipStream_t s) {
   dim3 grid(a.n_splits, a.n_kv, a.n_seqs);
   kern<<<grid, 64 * NW, lds, s>>>(a.qkv, a.q, a.cos_t, a.sin_t, a.style, a.k, a.v, a.out, a.tok_pos, a.bt,
                                   a.bt_stride, a.n_heads, a.n_kv, a.sl2, a.window, a.n_splits, a.ws, a.qkv_terms,
-                                  a.qkv_stride, a.sinks);
+                                  a.qkv_stride, a.sinks, a.keep_first, a.cap, a.cap_pre);
   if (a.n_splits > 1) attn_decode_combine_kernel<D><<<a.n_seqs * a.n_heads, D, 0, s>>>(a.ws, a.out, a.n_splits, a.sinks, a.n_heads);
   return 0;
 }
@@ -1126,7 +1140,9 @@ static int dispatch_decode(const DecodeArgs& a, int head_dim, hipStream_t s, con
   RB_REQUIRE(group <= 16, "%s: %d query heads per kv head not supported (at most 16; use rb_attention_generic)", who,
              group);
   RB_REQUIRE(g_decode_mfma != 2 || vector_ok, "%s: the vector kernel is built for 1, 2, 4 or 8 heads per kv head", who);
-  if (g_decode_mfma == 1 || !vector_ok || (g_decode_mfma == 0 && group > 1)) {
+  const bool opts = a.keep_first > 0 || a.cap > 0.f;      // kept first keys and capped scores: the matrix-core kernel has them
+  RB_REQUIRE(!opts || g_decode_mfma != 2, "%s: kept first keys and capped scores need the matrix-core kernel", who);
+  if (opts || g_decode_mfma == 1 || !vector_ok || (g_decode_mfma == 0 && group > 1)) {
     const int rc = head_dim == 128 ? launch_decode_mfma<128, FUSED>(a, s) : launch_decode_mfma<64, FUSED>(a, s);
     if (rc) return rc;
     RB_LAUNCH_CHECK();
@@ -1153,6 +1169,23 @@ extern "C" int rb_attention_decode_bf16(const void* q, const void* k_pages, cons
                                         int window, int n_splits, float* workspace, void* stream) {
   return rb_attention_decode_bf16_sinks(q, k_pages, v_pages, out, tok_pos, block_table, bt_stride, n_seqs, n_heads,
                                         n_kv_heads, head_dim, scale, window, n_splits, workspace, nullptr, stream);
+}
+
+extern "C" int rb_attention_decode_bf16_opts(const void* q, const void* k_pages, const void* v_pages, void* out,
+                                             const int32_t* tok_pos, const int32_t* block_table, int bt_stride, int n_seqs,
+                                             int n_heads, int n_kv_heads, int head_dim, float scale, int window, int keep_first,
+                                             float softcap, int n_splits, float* workspace, const float* sinks, void* stream) {
+  RB_RECORDED(rb_attention_decode_bf16_opts(q, k_pages, v_pages, out, tok_pos, block_table, bt_stride, n_seqs, n_heads,
+                                            n_kv_heads, head_dim, scale, window, keep_first, softcap, n_splits, workspace, sinks,
+                                            stream));
+  RB_REQUIRE(keep_first >= 0 && softcap >= 0.f, "rb_attention_decode_bf16: negative keep_first or softcap");
+  DecodeArgs a = {nullptr, (const bf16_t*)q, nullptr, nullptr, 0, (bf16_t*)k_pages, (bf16_t*)v_pages, (bf16_t*)out,
+                  tok_pos, block_table, bt_stride, n_seqs, n_heads, n_kv_heads, softcap > 0.f ? LOG2E : scale * LOG2E, window,
+                  n_splits, workspace, 1, 0, sinks};
+  a.keep_first = window > 0 ? keep_first : 0;
+  a.cap = softcap;
+  a.cap_pre = softcap > 0.f ? scale / softcap : 0.f;
+  return dispatch_decode<false>(a, head_dim, (hipStream_t)stream, "rb_attention_decode_bf16");
 }
 
 extern "C" int rb_attention_decode_bf16_sinks(const void* q, const void* k_pages, const void* v_pages, void* out,

@@ -52,7 +52,7 @@ extern "C" int rb_gemm_bf16(const void* a, const void* w, int w_layout, void* c,
 extern "C" int rb_gemm_bf16_act(const void* a, const void* w, int w_layout, void* c, int dtype_out, int epilogue,
                                 const float* act, int m, int n, int k, float* workspace, void* stream) {
   RB_RECORDED(rb_gemm_bf16_act(a, w, w_layout, c, dtype_out, epilogue, act, m, n, k, workspace, stream));
-  RB_REQUIRE(act == nullptr || epilogue == 0, "rb_gemm_bf16: an activation goes with epilogue 0, not %d", epilogue);
+  RB_REQUIRE(act == nullptr || epilogue <= 1, "rb_gemm_bf16: an activation goes with epilogue 0, a gate's numbers with 1, not %d", epilogue);
   RB_REQUIRE(m >= 0 && n > 0 && k > 0, "rb_gemm_bf16: bad sizes M=%d N=%d K=%d", m, n, k);
   RB_REQUIRE(layout_ok(w_layout, n, k), "rb_gemm_bf16: W layout %d with N=%d K=%d (fragment-major needs N %% 16 == 0, K %% 64 == 0)",
              w_layout, n, k);

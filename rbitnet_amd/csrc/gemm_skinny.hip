@@ -328,6 +328,7 @@ __global__ __launch_bounds__(512) void gemm_skinny_kernel(const bf16_t* __restri
                             n0 / 16 + rt, kq, fa);
   } else {
     const int half_n = n / 2;
+    const GatePair gp = gate_pair(fa.act);
 #pragma unroll
     for (int rt = 0; rt + 1 < R; rt += 2)
 #pragma unroll
@@ -338,7 +339,7 @@ __global__ __launch_bounds__(512) void gemm_skinny_kernel(const bf16_t* __restri
         TO* dst = c + (size_t)mm * half_n + nn;
 #pragma unroll
         for (int i = 0; i < 4; ++i)
-          if (nn + i < half_n) Num<TO>::store(dst + i, silu_f32(acc[rt][cb][i]) * acc[rt + 1][cb][i]);
+          if (nn + i < half_n) Num<TO>::store(dst + i, gated_value(acc[rt][cb][i], acc[rt + 1][cb][i], gp));
       }
   }
 }
@@ -351,7 +352,7 @@ extern "C" void rb_tune(int r, int waves) {       // experiments only; 0 = the b
 
 static FoldArgs fold_args(const GemmTokens& x, const GemmAfter& after) {
   return FoldArgs{x.squares, x.rows, x.eps, after.gain, after.gained, after.squares, after.w_frag ? 1 : 0,
-                  after.epilogue == 0 ? after.act : nullptr};
+                  after.epilogue <= 1 ? after.act : nullptr};
 }
 
 template <int MB, int R, int U, bool FAST, int EPI, typename TO, bool SCALED>
@@ -602,6 +603,7 @@ __global__ __launch_bounds__(512) void gemm_resident_kernel(const bf16_t* __rest
       for (int cb = 0; cb < MB; ++cb) gate[cb] = acc[cb];
     } else {
       const int half_n = n / 2;
+      const GatePair gp = gate_pair(fa.act);
 #pragma unroll
       for (int cb = 0; cb < MB; ++cb) {
         const int mm = 16 * cb + r;
@@ -610,7 +612,7 @@ __global__ __launch_bounds__(512) void gemm_resident_kernel(const bf16_t* __rest
         TO* dst = cpart + (size_t)mm * half_n + nn;
 #pragma unroll
         for (int i = 0; i < 4; ++i)
-          if (nn + i < half_n) Num<TO>::store(dst + i, silu_f32(gate[cb][i]) * acc[cb][i]);
+          if (nn + i < half_n) Num<TO>::store(dst + i, gated_value(gate[cb][i], acc[cb][i], gp));
       }
     }
   };

@@ -55,7 +55,7 @@ __device__ __forceinline__ bool tile_of_workgroup(int m_tiles, int n_tiles, int*
 template <int EPI, typename TO>
 __device__ __forceinline__ void store_piece(const f32x16_t& acc, TO* __restrict__ c, float* __restrict__ slab,
                                             int first_row, int l32, int mbase, int m, int n, bool has_act = false,
-                                            float ap = 0.f, float an = 0.f) {
+                                            float ap = 0.f, float an = 0.f, GatePair gp = GatePair{0.f, 0.f}) {
   if (EPI == 0) {
     const int nn = first_row + l32;
     if (nn >= n) return;
@@ -79,7 +79,7 @@ __device__ __forceinline__ void store_piece(const f32x16_t& acc, TO* __restrict_
       const float got = __shfl_xor(give, 16);
       const int mm = mbase + 8 * (e / 4) + (e % 4) + (upper ? 1 : 0);
       const float gate = upper ? got : mine, up = upper ? mine : got;
-      if (mm < m && col < half_n) Num<TO>::store(c + (size_t)mm * half_n + col, silu_f32(gate) * up);
+      if (mm < m && col < half_n) Num<TO>::store(c + (size_t)mm * half_n + col, gated_value(gate, up, gp));
     }
   }
 }
@@ -243,11 +243,12 @@ __global__ __launch_bounds__(64 * (BN / WN) * (BM / WM)) void gemm_tiled_kernel(
   const bool has_act = EPI == 0 && act != nullptr;
   XieluPair xa = {0.f, 0.f};
   if (has_act) xa = xielu_pair(act);
+  const GatePair gp = gate_pair(EPI == 1 ? act : nullptr);
 #pragma unroll
   for (int i = 0; i < TN; ++i)
 #pragma unroll
     for (int j = 0; j < TM; ++j)
-      store_piece<EPI, TO>(acc[i][j], c, nullptr, n0 + wn0 + 32 * i, l32, m0 + wm0 + 32 * j + 4 * g, m, n, has_act, xa.ap, xa.an);
+      store_piece<EPI, TO>(acc[i][j], c, nullptr, n0 + wn0 + 32 * i, l32, m0 + wm0 + 32 * j + 4 * g, m, n, has_act, xa.ap, xa.an, gp);
 }
 
 // ---------------------------------------------------------------------------------------
@@ -503,6 +504,7 @@ __global__ __launch_bounds__(64 * (BN / WN) * (BM / WM)) void gemm_dma_kernel(co
     constexpr int CH = HC / 8;              // 16-byte chunks of a row
     static_assert((size_t)BM * LD <= (size_t)S * STAGE, "the tile's outputs do not fit the stages");
     const int half_n = n / 2;
+    const GatePair gp = gate_pair(act);
     __syncthreads();                        // everyone has read its last fragments
     const bool upper = (l32 & 16) != 0;
 #pragma unroll
@@ -518,7 +520,7 @@ __global__ __launch_bounds__(64 * (BN / WN) * (BM / WM)) void gemm_dma_kernel(co
           const float give = upper ? acc[i][j][e] : acc[i][j][e + 1];
           const float got = __shfl_xor(give, 16);
           const float gate = upper ? got : mine, up = upper ? mine : got;
-          dst[(size_t)(8 * (e / 4) + (e % 4)) * LD] = f32_to_bf16(silu_f32(gate) * up);
+          dst[(size_t)(8 * (e / 4) + (e % 4)) * LD] = f32_to_bf16(gated_value(gate, up, gp));
         }
       }
     __syncthreads();
@@ -541,11 +543,12 @@ __global__ __launch_bounds__(64 * (BN / WN) * (BM / WM)) void gemm_dma_kernel(co
   const bool has_act = EPI == 0 && act != nullptr && slab == nullptr;      // slices leave the activation to the sum of the slabs
   XieluPair xa = {0.f, 0.f};
   if (has_act) xa = xielu_pair(act);
+  const GatePair gp = gate_pair(EPI == 1 ? act : nullptr);
 #pragma unroll
   for (int i = 0; i < TN; ++i)
 #pragma unroll
     for (int j = 0; j < TM; ++j)
-      store_piece<EPI, TO>(acc[i][j], c, slab, n0 + wn0 + 32 * i, l32, m0 + wm0 + 32 * j + 4 * g, m, n, has_act, xa.ap, xa.an);
+      store_piece<EPI, TO>(acc[i][j], c, slab, n0 + wn0 + 32 * i, l32, m0 + wm0 + 32 * j + 4 * g, m, n, has_act, xa.ap, xa.an, gp);
 }
 
 template <int BN, int BM, int WN, int WM, int BK, int S, int EPI, typename TO, bool WF>
@@ -570,12 +573,12 @@ static int launch_dma_cfg(const bf16_t* x, const bf16_t* w, void* c, int m, int 
     configured = true;
   }
   const dim3 grid((unsigned)((tiles + 7) / 8 * 8), (unsigned)parts);
-  RB_REQUIRE(act == nullptr || (EPI == 0 && c != nullptr), "rb_gemm_bf16: internal: an activation goes with epilogue 0 and an output");
+  RB_REQUIRE(act == nullptr || (EPI <= 1 && c != nullptr), "rb_gemm_bf16: internal: an activation or a gate's numbers go with epilogues 0 and 1 and an output");
   kern<<<grid, 64 * (BN / WN) * (BM / WM), lds, s>>>(x, w, (TO*)c, parts > 1 ? slabs : nullptr, m, n, k, m_tiles,
                                                       n_tiles, k / BK / parts, act);
   if (parts > 1 && c != nullptr) {      // without c the caller adds the slabs up itself
     const size_t count = (size_t)m * n;
-    gemm_sum_slabs_kernel<TO><<<(unsigned)((count + 255) / 256), 256, 0, s>>>(slabs, (TO*)c, parts, count, act);
+    gemm_sum_slabs_kernel<TO><<<(unsigned)((count + 255) / 256), 256, 0, s>>>(slabs, (TO*)c, parts, count, EPI == 0 ? act : nullptr);
   }
   return 0;
 }
@@ -599,7 +602,7 @@ static int launch_tiled_cfg(const bf16_t* x, const bf16_t* w, void* c, int m, in
     configured[tail] = true;
   }
   const int grid = (int)((tiles + 7) / 8 * 8);
-  kern<<<grid, 64 * (BN / WN) * (BM / WM), lds, s>>>(x, w, (TO*)c, m, n, k, m_tiles, n_tiles, EPI == 0 ? act : nullptr);
+  kern<<<grid, 64 * (BN / WN) * (BM / WM), lds, s>>>(x, w, (TO*)c, m, n, k, m_tiles, n_tiles, EPI <= 1 ? act : nullptr);
   return 0;
 }
 
@@ -763,7 +766,7 @@ int gemm_tiled_parts(int m, int n, int k, int epilogue) {
 
 int gemm_tiled_launch(const bf16_t* x, const bf16_t* w, bool w_frag, void* c, float* workspace, int dtype_out,
                       int epilogue, int m, int n, int k, hipStream_t s, const float* act) {
-  RB_REQUIRE(act == nullptr || epilogue == 0, "rb_gemm_bf16: an activation goes with epilogue 0");
+  RB_REQUIRE(act == nullptr || epilogue <= 1, "rb_gemm_bf16: an activation goes with epilogue 0, a gate's numbers with epilogue 1");
   if (w_frag) return RB_BY_OUTPUT(launch_planned, true, x, w, c, workspace, m, n, k, s, act);
   return RB_BY_OUTPUT(launch_planned, false, x, w, c, workspace, m, n, k, s, act);
 }

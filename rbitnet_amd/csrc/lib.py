@@ -185,6 +185,7 @@ class Kernels:
             "rb_clamped_glu": [_P, _P, _I, _I, _I, _F, _F, _P],
             "rb_tanh_cast": [_P, _P, _I, _L, _P],
             "rb_attention_prefill_bf16_opts": [_P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _I, _I, _F, _P, _P],
+            "rb_attention_decode_bf16_opts": [_P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _F, _I, _I, _F, _I, _P, _P, _P],
             "rb_attention_generic_opts": [_P, _P, _P, _P, _I, _P, _P, _P, _I, _I, _I, _I, _I, _F, _I, _I, _F, _P, _P],
             "rb_norm_rope_store": [_P, _L, _P, _P, _I, _P, _P, _F, _P, _P, _P, _I, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _P],
             "rb_sigmoid_gate": [_P, _I, _P, _L, _P],
@@ -312,7 +313,8 @@ class Kernels:
     def gemm_bf16(self, a: torch.Tensor, w: torch.Tensor, c: torch.Tensor, epilogue: int = 0,
                   w_frag: bool = False, act: Optional[torch.Tensor] = None) -> None:
         """w_frag: w [N, K] is stored fragment-major (`place_rows(..., frag=True)` writes that).
-        act (epilogue 0): the two numbers of xIELU, float32 [2]; the result is xIELU(a w^T)."""
+        act (epilogue 0): the two numbers of xIELU, float32 [2]; the result is xIELU(a w^T).  act (epilogue 1): the gated
+        pair's limit and alpha, float32 [2]; the result is g sigmoid(alpha g) (u + 1) with g and u limited."""
         m, k = a.shape
         n = w.shape[0]
         _check(a, "a", torch.bfloat16)
@@ -322,8 +324,8 @@ class Kernels:
         workspace = torch.empty(need, dtype=torch.float32, device=a.device) if need else None
         if act is not None:
             _check(act, "act", torch.float32, (2,))
-            if epilogue != 0:
-                raise KernelError("gemm_bf16: an activation goes with epilogue 0")
+            if epilogue not in (0, 1):
+                raise KernelError("gemm_bf16: an activation goes with epilogue 0, a gate's numbers with epilogue 1")
         self._ok(self._lib.rb_gemm_bf16_act(_ptr(a), _ptr(w), int(bool(w_frag)), _ptr(c), dtype_code(c.dtype), int(epilogue),
                                             _ptr(act), m, n, k, _ptr(workspace), self._stream()))
 
@@ -414,7 +416,7 @@ class Kernels:
                                                           float(softcap or 0.0), _ptr(sinks), self._stream()))
 
     def attention_decode_bf16(self, q, k_pages, v_pages, out, tok_pos, block_table, n_heads, n_kv, head_dim,
-                              scale, window, n_splits, workspace, sinks=None) -> None:
+                              scale, window, n_splits, workspace, sinks=None, keep_first: int = 0, softcap: float = 0.0) -> None:
         n = q.shape[0]
         _check(q, "q", torch.bfloat16, (n, n_heads, head_dim))
         _check(k_pages, "k_pages", torch.bfloat16)
@@ -429,6 +431,13 @@ class Kernels:
             raise KernelError("decode attention workspace too small")
         if sinks is not None:
             _check(sinks, "sinks", torch.float32, (n_heads,))
+        if keep_first or softcap:
+            self._ok(self._lib.rb_attention_decode_bf16_opts(_ptr(q), _ptr(k_pages), _ptr(v_pages), _ptr(out), _ptr(tok_pos),
+                                                             _ptr(block_table), block_table.shape[1], n, n_heads, n_kv,
+                                                             head_dim, float(scale), int(window or 0), int(keep_first or 0),
+                                                             float(softcap or 0.0), int(n_splits), _ptr(workspace), _ptr(sinks),
+                                                             self._stream()))
+            return
         self._ok(self._lib.rb_attention_decode_bf16_sinks(_ptr(q), _ptr(k_pages), _ptr(v_pages), _ptr(out), _ptr(tok_pos),
                                                           _ptr(block_table), block_table.shape[1], n, n_heads, n_kv,
                                                           head_dim, float(scale), int(window or 0), int(n_splits),
@@ -970,7 +979,9 @@ class Kernels:
         """proj [T, q_rank + kv_rank] float32: the two down-projections; cq [T, q_rank] and the pages
         [*, 1, 64, kv_rank] get their RMS norms (kv_rank 0: no latent is stored)."""
         n, width = proj.shape
-        _check(proj, "proj", torch.float32, (n, q_rank + kv_rank))
+        _check(proj, "proj", torch.float32)
+        if width < q_rank + kv_rank:
+            raise KernelError("latent_norm_store: rows too short for the two down-projections")
         if q_rank:
             _check(q_gain, "q_gain", torch.float32, (q_rank,))
             _check(cq, "cq", dtype, (n, q_rank))
@@ -1199,7 +1210,9 @@ class Kernels:
         norms, the pages also the last `rot` numbers rotated by the position, behind the latent, and zeros up to W."""
         n, width = proj.shape
         has_kv = kv_rank > 0
-        _check(proj, "proj", torch.float32, (n, q_rank + ((kv_rank + rot) if has_kv else 0)))
+        _check(proj, "proj", torch.float32)
+        if width < q_rank + ((kv_rank + rot) if has_kv else 0):
+            raise KernelError("latent_norm_rope_store: rows too short for the down-projections and the rotated part")
         _check(q_gain, "q_gain", torch.float32, (q_rank,))
         _check(cq, "cq", dtype, (n, q_rank))
         page_width = 0

@@ -49,6 +49,27 @@ __device__ __forceinline__ float silu_f32(float v) {
   return v * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-1.44269504088896341f * v));
 }
 
+// The gated pair of a product's epilogue 1: silu(gate) * up, or, with limits (two numbers (limit, alpha) given with the
+// product, limit > 0): g = min(gate, limit), u = clamp(up, -limit, limit), g * sigmoid(alpha g) * (u + 1).
+struct GatePair {
+  float lim, na;        // the limit (0: none) and -alpha * log2(e)
+};
+__device__ __forceinline__ GatePair gate_pair(const float* __restrict__ act) {
+  GatePair r = {0.f, 0.f};
+  if (act) {
+    r.lim = act[0];
+    r.na = -1.44269504088896341f * act[1];
+  }
+  return r;
+}
+__device__ __forceinline__ float gated_value(float gate, float up, const GatePair& gp) {
+  if (gp.lim > 0.f) {
+    const float g = fminf(gate, gp.lim), u = fminf(fmaxf(up, -gp.lim), gp.lim);
+    return g * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(gp.na * g)) * (u + 1.0f);
+  }
+  return silu_f32(gate) * up;
+}
+
 // ---- memory -> LDS without registers (global_load_lds_dwordx4): the 64 lanes of a wave fetch
 // 16 bytes each from base + their byte offset, and the 1 KB lands at the given LDS address in
 // lane order.  The instruction is inline assembly, so the compiler neither counts nor waits

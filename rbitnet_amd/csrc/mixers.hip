@@ -366,12 +366,16 @@ extern "C" int rb_norm_rope_store(const float* qkv, long long row_width, const f
   RB_REQUIRE(row_width >= need, "rb_norm_rope_store: rows of %lld numbers, %lld needed", row_width, need);
   if (n_tokens == 0) return 0;
   hipStream_t s = (hipStream_t)stream;
+  // a wave a head, up to 16 waves a token: a wave's heads are a chain of trips to memory
+  int waves = n_heads + (k_pages ? n_kv_heads : 0);
+  waves = waves > 16 ? 16 : (waves < 4 ? 4 : waves);
+  const int threads = RB_WAVE * waves;
   if (cache_dtype == RB_F32)
-    norm_rope_store_kernel<float><<<n_tokens, 256, 0, s>>>(qkv, (size_t)row_width, cos, sin, rot, q_norm, k_norm, eps, (float*)q_out,
+    norm_rope_store_kernel<float><<<n_tokens, threads, 0, s>>>(qkv, (size_t)row_width, cos, sin, rot, q_norm, k_norm, eps, (float*)q_out,
                                                            (float*)k_pages, (float*)v_pages, tok_pos, tok_seq, block_table,
                                                            bt_stride, n_heads, n_kv_heads, dim, vdim, pad);
   else if (cache_dtype == RB_BF16)
-    norm_rope_store_kernel<bf16_t><<<n_tokens, 256, 0, s>>>(qkv, (size_t)row_width, cos, sin, rot, q_norm, k_norm, eps,
+    norm_rope_store_kernel<bf16_t><<<n_tokens, threads, 0, s>>>(qkv, (size_t)row_width, cos, sin, rot, q_norm, k_norm, eps,
                                                             (bf16_t*)q_out, (bf16_t*)k_pages, (bf16_t*)v_pages, tok_pos, tok_seq,
                                                             block_table, bt_stride, n_heads, n_kv_heads, dim, vdim, pad);
   else

@@ -112,8 +112,9 @@ class DenseGelu(DenseAct):
 class ClampedGLU(Part):
     """A gated feed-forward with limits on both branches:
         g = min(Wgate h, limit),  u = clamp(Wup h, -limit, limit);  out = Wdown (g * sigmoid(alpha * g) * (u + 1))
-    (the unit of the routed experts, as a dense layer).  Gate and up are one product with float32 sums; limits, gate and
-    the rounding to the compute dtype are one kernel on them.
+    (the unit of the routed experts, as a dense layer).  Gate and up are one product; on the matrix cores limits and gate
+    are applied in that product's epilogue (gate and up rows interleaved, as for the SiLU gate), elsewhere by a kernel on
+    its float32 sums.
     Parameters: intermediate_size, limit (None or <= 0: no limits), alpha (1.702), names ({"gate", "up", "down"})."""
     graph_safe = True
     plan_safe = True
@@ -125,6 +126,7 @@ class ClampedGLU(Part):
         self.alpha = float(params.get("alpha", 1.702))
         self.names = dict({"gate": "gate", "up": "up", "down": "down"}, **(params.get("names") or {}))
         self.hidden = env.hidden_size
+        self.fused = self.limit > 0 and can_fuse_gate(env.dtype, self.hidden, self.ff) and not getattr(env, "generic_only", False)
 
     def tensor_specs(self) -> Dict[str, TensorSpec]:
         return {self.names["gate"]: TensorSpec((self.ff, self.hidden)), self.names["up"]: TensorSpec((self.ff, self.hidden)),
@@ -132,16 +134,20 @@ class ClampedGLU(Part):
 
     def load(self, tensors: Dict[str, torch.Tensor]) -> None:
         allowed = not getattr(self.env, "generic_only", False)
-        self.w_gate_up = pack_gate_up(self.env.lib, tensors[self.names["gate"]], tensors[self.names["up"]], False, allowed)
+        self.w_gate_up = pack_gate_up(self.env.lib, tensors[self.names["gate"]], tensors[self.names["up"]], self.fused, allowed)
+        self.gate_numbers = torch.tensor([self.limit, self.alpha], dtype=torch.float32, device=tensors[self.names["gate"]].device)
         down = tensors[self.names["down"]]
         self.w_down = pack_rows(self.env.lib, [(down, 0, None, None)], down.shape[0], down.shape[1], down.dtype, down.device,
                                 allowed)
 
     def forward(self, h, ctx=None, stream: Optional[torch.Tensor] = None, next_norm=None):
         lib = self.env.lib
-        gu = linear(lib, h, self.w_gate_up, torch.float32)
-        t = torch.empty((h.shape[0], self.ff), dtype=self.env.dtype, device=gu.device)
-        lib.clamped_glu(gu, t, self.limit, self.alpha)
+        if self.fused:
+            t = gated_linear(lib, h, self.w_gate_up, self.ff, True, gate=self.gate_numbers)
+        else:
+            gu = linear(lib, h, self.w_gate_up, torch.float32)
+            t = torch.empty((h.shape[0], self.ff), dtype=self.env.dtype, device=gu.device)
+            lib.clamped_glu(gu, t, self.limit, self.alpha)
         return linear(lib, t, self.w_down, torch.float32)
 
 

@@ -110,6 +110,13 @@ class LatentAttention(Part):
         pieces = [(tensors[n["dq"]], 0, None, None)] + ([(tensors[n["dkv"]], self.q_rank, None, None)] if owns else [])
         first = tensors[n["dq"]]
         rows = self.q_rank + ((self.kv_rank + self.rot) if owns else 0)
+        self.gate_col = rows
+        if self.has_gate:       # the gate's rows ride in the same product (behind the others, up to a multiple of 16 with zeros)
+            g = tensors[n["gate"]]
+            full = torch.zeros(((rows + self.heads + 15) // 16 * 16 - rows, self.hidden), dtype=g.dtype, device=g.device)
+            full[:self.heads] = g
+            pieces.append((full, rows, None, None))
+            rows += full.shape[0]
         self.w_down = pack_rows(lib, pieces, rows, self.hidden, first.dtype, first.device, allowed)
         self.q_gain = tensors[n["dq_norm"]]
         self.kv_gain = tensors[n["dkv_norm"]] if owns else None
@@ -120,13 +127,6 @@ class LatentAttention(Part):
         self.w_uk = tensors[n["uk"]].view(self.heads, self.dim, self.kv_rank).contiguous()
         self.w_uv = tensors[n["uv"]].view(self.heads, self.vdim, self.kv_rank).transpose(1, 2).contiguous()
         self.sink = tensors[n["sink"]] if self.has_sink else None
-        self.w_gate = None
-        if self.has_gate:       # rows up to a multiple of 16 (zeros), so that the product's kernels find whole tiles
-            g = tensors[n["gate"]]
-            rows = (self.heads + 15) // 16 * 16
-            full = torch.zeros((rows, self.hidden), dtype=g.dtype, device=g.device)
-            full[:self.heads] = g
-            self.w_gate = pack_rows(lib, [(full, 0, None, None)], rows, self.hidden, g.dtype, g.device, allowed)
 
     def cache_request(self) -> Optional[CacheRequest]:
         if self.cache_from is not None:
@@ -174,7 +174,7 @@ class LatentAttention(Part):
         else:
             lib.heads_linear(ol, self.w_uv, o)
         if self.has_gate:
-            lib.head_gate(o, linear(lib, h, self.w_gate, torch.float32), 0, self.heads, self.vdim)
+            lib.head_gate(o, down, self.gate_col, self.heads, self.vdim)
         return linear(lib, o, self.w_o, torch.float32)
 
 

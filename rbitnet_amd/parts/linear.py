@@ -167,8 +167,9 @@ def pack_gate_up(lib, gate: torch.Tensor, up: torch.Tensor, fused: bool, frag_al
     return pack_rows(lib, pieces, 2 * ff, k, gate.dtype, gate.device, frag_allowed)
 
 
-def gated_linear(lib, x, w_packed, ff: int, fused: bool) -> torch.Tensor:
-    """silu(x Wg^T) * (x Wu^T) -> [M, ff] in x's dtype."""
+def gated_linear(lib, x, w_packed, ff: int, fused: bool, gate: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """silu(x Wg^T) * (x Wu^T) -> [M, ff] in x's dtype.  gate (fused only; float32 [2] = (limit, alpha)): the gated pair with
+    limits instead, g sigmoid(alpha g) (u + 1) with g = min(x Wg^T, limit), u = clamp(x Wu^T, -limit, limit)."""
     m = x.shape[0]
     out = torch.empty((m, ff), dtype=x.dtype, device=x.device)
     if m == 0:
@@ -180,7 +181,7 @@ def gated_linear(lib, x, w_packed, ff: int, fused: bool) -> torch.Tensor:
         x = x.tensor()
     if fused:
         wd, frag = _data(w_packed)
-        lib.gemm_bf16(x, wd, out, 1, w_frag=frag)
+        lib.gemm_bf16(x, wd, out, 1, w_frag=frag, act=gate)
     else:
         gu = linear(lib, x, w_packed, torch.float32)
         lib.swiglu(gu, out)

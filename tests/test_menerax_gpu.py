@@ -246,6 +246,27 @@ def test_windowed_attention_whole_in_pieces_and_token_by_token(lib, p, dtype):
         assert _close(torch.cat(_run_mixer(lib, part, x, cuts, dtype)), want, dtype), cuts
 
 
+@pytest.mark.parametrize("splits", [1, 3, 16])
+def test_long_decoding_past_the_window_with_the_pages_dealt_to_several_workgroups(lib, splits):
+    """1,300 tokens, the last 60 one by one: the window's pages and the kept tokens' pages are far apart, and the step's
+    workgroups share them out (the number of shares forced, as a long context would choose it)."""
+    from rbitnet_amd.engine import context as C
+    hidden, t_len = 64, 1300
+    p = _left(4, 2, 64, 64, 3, 32, 1e4, 0.125, softcap=20.0, mask={"size": 200, "keep_first": 70})
+    w = _left_weights(hidden, p, seed=11)
+    x = _bf(torch.randn(t_len, hidden, dtype=F64))
+    want = P.windowed_attention(x, w, p, EPS)
+    part = _left_part(lib, hidden, p, torch.bfloat16)
+    part.load(_place(part, w, torch.bfloat16))
+    C.FORCED_DECODE_SPLITS = splits
+    try:
+        got = torch.cat(_run_mixer(lib, part, x, [t_len - 60] + [1] * 60, torch.bfloat16, pages=22))
+    finally:
+        C.FORCED_DECODE_SPLITS = None
+    assert _close(got, want, torch.bfloat16)
+    assert _close(got[-60:], want[-60:], torch.bfloat16)
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("window,keep,dim,vdim", [(40, 20, 16, 12), (64, 64, 64, 64), (65, 3, 64, 128), (7, 70, 8, 12)])
 def test_a_key_that_stands_out_at_every_edge_of_the_mask(lib, dtype, window, keep, dim, vdim):
