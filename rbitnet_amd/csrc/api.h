@@ -317,6 +317,8 @@ int rb_attention_generic_opts(const void* q, const void* k_pages, const void* v_
                               int n_tokens, int n_heads, int n_kv_heads, int head_dim, float scale, int window, int keep_first,
                               float softcap, const float* sinks, void* stream);
 // The matrix-core kernels with the same two choices (see rb_attention_prefill_bf16_sinks, rb_attention_decode_bf16_sinks).
+// The decode entry point also takes more than 16 query heads on a key/value head: they run as the fewest groups of equal
+// size that hold at most 16 each, every group reading that head's pages.
 int rb_attention_prefill_bf16_opts(const void* q, const void* k_pages, const void* v_pages, void* out,
                                    const int32_t* cu_seqlens, const int32_t* past_len, const int32_t* block_table,
                                    int bt_stride, int n_seqs, int max_q_len, int n_heads, int n_kv_heads, int head_dim,

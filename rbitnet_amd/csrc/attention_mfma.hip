@@ -719,7 +719,9 @@ __global__ __launch_bounds__(64 * NW) void attn_decode_mfma_kernel(
     const float* __restrict__ sin_t, int style, bf16_t* k_pages, bf16_t* v_pages, bf16_t* __restrict__ out,
     const int32_t* __restrict__ tok_pos, const int32_t* __restrict__ block_table, int bt_stride, int n_heads,
     int n_kv, float scale_log2, int window, int n_splits, float* __restrict__ ws, int qkv_terms, size_t qkv_stride,
-    const float* __restrict__ sinks, int keep_first, float cap, float cap_pre) {
+    const float* __restrict__ sinks, int keep_first, float cap, float cap_pre, int kv_rep) {
+  // kv_rep > 1: n_kv counts every key/value head kv_rep times (head kvh reads the pages of head kvh / kv_rep), so that more
+  // than 16 query heads on one key/value head run as several groups of at most 16.
   // keep_first (with a window): the first keep_first keys stay visible behind the window; their pages are walked before the
   // window's.  cap > 0: a raw score s becomes cap * tanh(s * cap_pre) (cap_pre = scale / cap), and scale_log2 is log2(e).
   constexpr int KS = D / 32;          // depth steps of the score product
@@ -771,7 +773,7 @@ __global__ __launch_bounds__(64 * NW) void attn_decode_mfma_kernel(
   // every load of a page.
   constexpr bool v_once = ONCE >= 1, k_once = ONCE >= 2;
   auto ask_values = [&](int page) {        // into this wave's area of LDS
-    const bf16_t* rows = v_pages + ((size_t)page * n_kv + kvh) * RB_PAGE * D;
+    const bf16_t* rows = v_pages + ((size_t)page * (n_kv / kv_rep) + kvh / kv_rep) * RB_PAGE * D;
 #pragma unroll
     for (int i = 0; i < VI; ++i) {
       const int key = i * RPI + lane / CPR;
@@ -781,7 +783,7 @@ __global__ __launch_bounds__(64 * NW) void attn_decode_mfma_kernel(
     }
   };
   auto ask_keys = [&](int page) {          // into kf_next
-    const bf16_t* rows = k_pages + ((size_t)page * n_kv + kvh) * RB_PAGE * D;
+    const bf16_t* rows = k_pages + ((size_t)page * (n_kv / kv_rep) + kvh / kv_rep) * RB_PAGE * D;
 #pragma unroll
     for (int t = 0; t < 4; ++t)
 #pragma unroll
@@ -1060,6 +1062,7 @@ struct DecodeArgs {
   int keep_first = 0;     // with a window: the first keys that stay visible behind it
   float cap = 0.f;        // > 0: scores capped at cap * tanh(score / cap); sl2 is then log2(e) and cap_pre scale / cap
   float cap_pre = 0.f;
+  int kv_rep = 1;         // n_kv counts every key/value head this many times (groups of at most 16 query heads on one of them)
 };
 
 template <int D, int G, bool FUSED>
@@ -1085,7 +1088,7 @@ static int launch_decode_mfma_nw(const DecodeArgs& a, hipStream_t s) {
   dim3 grid(a.n_splits, a.n_kv, a.n_seqs);
   kern<<<grid, 64 * NW, lds, s>>>(a.qkv, a.q, a.cos_t, a.sin_t, a.style, a.k, a.v, a.out, a.tok_pos, a.bt,
                                   a.bt_stride, a.n_heads, a.n_kv, a.sl2, a.window, a.n_splits, a.ws, a.qkv_terms,
-                                  a.qkv_stride, a.sinks, a.keep_first, a.cap, a.cap_pre);
+                                  a.qkv_stride, a.sinks, a.keep_first, a.cap, a.cap_pre, a.kv_rep);
   if (a.n_splits > 1) attn_decode_combine_kernel<D><<<a.n_seqs * a.n_heads, D, 0, s>>>(a.ws, a.out, a.n_splits, a.sinks, a.n_heads);
   return 0;
 }
@@ -1140,7 +1143,7 @@ static int dispatch_decode(const DecodeArgs& a, int head_dim, hipStream_t s, con
   RB_REQUIRE(group <= 16, "%s: %d query heads per kv head not supported (at most 16; use rb_attention_generic)", who,
              group);
   RB_REQUIRE(g_decode_mfma != 2 || vector_ok, "%s: the vector kernel is built for 1, 2, 4 or 8 heads per kv head", who);
-  const bool opts = a.keep_first > 0 || a.cap > 0.f;      // kept first keys and capped scores: the matrix-core kernel has them
+  const bool opts = a.keep_first > 0 || a.cap > 0.f || a.kv_rep > 1;      // kept first keys, capped scores, repeated kv heads: the matrix-core kernel has them
   RB_REQUIRE(!opts || g_decode_mfma != 2, "%s: kept first keys and capped scores need the matrix-core kernel", who);
   if (opts || g_decode_mfma == 1 || !vector_ok || (g_decode_mfma == 0 && group > 1)) {
     const int rc = head_dim == 128 ? launch_decode_mfma<128, FUSED>(a, s) : launch_decode_mfma<64, FUSED>(a, s);
@@ -1185,6 +1188,14 @@ extern "C" int rb_attention_decode_bf16_opts(const void* q, const void* k_pages,
   a.keep_first = window > 0 ? keep_first : 0;
   a.cap = softcap;
   a.cap_pre = softcap > 0.f ? scale / softcap : 0.f;
+  // more than 16 query heads on a key/value head: the fewest groups of equal size that hold at most 16 each
+  if (n_kv_heads > 0 && n_heads % n_kv_heads == 0) {
+    const int group = n_heads / n_kv_heads;
+    int reps = 1;
+    while (reps < group && (group % reps != 0 || group / reps > 16)) ++reps;
+    a.kv_rep = reps;
+    a.n_kv = n_kv_heads * reps;
+  }
   return dispatch_decode<false>(a, head_dim, (hipStream_t)stream, "rb_attention_decode_bf16");
 }
 

@@ -17,7 +17,9 @@ __global__ void latent_norm_store_kernel(const float* __restrict__ proj, size_t 
                                          const float* __restrict__ q_gain, TC* __restrict__ cq, int kv_col, int kv_rank,
                                          const float* __restrict__ kv_gain, TC* __restrict__ pages, int page_width,
                                          const int32_t* __restrict__ tok_pos, const int32_t* __restrict__ tok_seq,
-                                         const int32_t* __restrict__ block_table, int bt_stride, float eps) {
+                                         const int32_t* __restrict__ block_table, int bt_stride, float eps, int rot_col = 0,
+                                         int rot = 0, const float* __restrict__ cos_t = nullptr,
+                                         const float* __restrict__ sin_t = nullptr, int style = 0) {
   __shared__ float scratch[16];
   const int t = blockIdx.x;
   const float* row = proj + (size_t)t * stride;
@@ -36,6 +38,22 @@ __global__ void latent_norm_store_kernel(const float* __restrict__ proj, size_t 
     for (int j = threadIdx.x; j < kv_rank; j += blockDim.x) ss = fmaf(src[j], src[j], ss);
     const float f = 1.0f / sqrtf(block_sum(ss, scratch) / (float)kv_rank + eps);
     for (int j = threadIdx.x; j < kv_rank; j += blockDim.x) Num<TC>::store(dst + j, src[j] * f * kv_gain[j]);
+    // behind the latent: the row's `rot` numbers at rot_col rotated by the position (not normed), then zeros up to page_width
+    if (page_width > kv_rank) {
+      const int half = rot / 2;
+      const float* rsrc = row + rot_col;
+      const float* cr = cos_t + (size_t)pos * half;
+      const float* sr = sin_t + (size_t)pos * half;
+      TC* rdst = dst + kv_rank;
+      for (int i = threadIdx.x; i < half; i += blockDim.x) {
+        const int a = style == 0 ? 2 * i : i, b = style == 0 ? 2 * i + 1 : i + half;
+        float y0, y1;
+        rotate_pair(rsrc[a], rsrc[b], cr[i], sr[i], y0, y1);
+        Num<TC>::store(rdst + a, y0);
+        Num<TC>::store(rdst + b, y1);
+      }
+      for (int i = rot + threadIdx.x; i < page_width - kv_rank; i += blockDim.x) Num<TC>::store(rdst + i, 0.f);
+    }
   }
 }
 
@@ -177,30 +195,8 @@ extern "C" int rb_heads_linear_strided(const void* x, int x_dtype, long long x_h
 // the latent c and, behind it, that rotated part: one key/value head of page_width >= kv_rank + rot numbers (the rest
 // zeros), and a query is [Wk^T q_unrotated, rotate(q_rotated)] in the same layout.
 // rb_latent_norm_store with that: the `rot` numbers at rot_col of a row of proj are rotated by the token's position
-// (style 0: 2i with 2i + 1; 1: i with i + rot / 2; cos, sin [positions, rot / 2]) and stored behind the latent.
-template <typename TC>
-__global__ void latent_rope_store_kernel(const float* __restrict__ proj, size_t stride, int kv_rank, int page_width, int rot_col,
-                                         int rot, const float* __restrict__ cos_t, const float* __restrict__ sin_t, int style,
-                                         TC* __restrict__ pages, const int32_t* __restrict__ tok_pos,
-                                         const int32_t* __restrict__ tok_seq, const int32_t* __restrict__ block_table, int bt_stride) {
-  const int t = blockIdx.x;
-  const int pos = tok_pos[t];
-  const int half = rot / 2;
-  const int page = block_table[(size_t)tok_seq[t] * bt_stride + pos / RB_PAGE];
-  TC* dst = pages + ((size_t)page * RB_PAGE + (size_t)(pos % RB_PAGE)) * page_width + kv_rank;
-  const float* src = proj + (size_t)t * stride + rot_col;
-  const float* cr = cos_t + (size_t)pos * half;
-  const float* sr = sin_t + (size_t)pos * half;
-  for (int i = threadIdx.x; i < half; i += blockDim.x) {
-    const int a = style == 0 ? 2 * i : i, b = style == 0 ? 2 * i + 1 : i + half;
-    float y0, y1;
-    rotate_pair(src[a], src[b], cr[i], sr[i], y0, y1);
-    Num<TC>::store(dst + a, y0);
-    Num<TC>::store(dst + b, y1);
-  }
-  for (int i = rot + threadIdx.x; i < page_width - kv_rank; i += blockDim.x) Num<TC>::store(dst + i, 0.f);
-}
-
+// (style 0: 2i with 2i + 1; 1: i with i + rot / 2; cos, sin [positions, rot / 2]) and stored behind the latent, by the same
+// launch.
 extern "C" int rb_latent_norm_rope_store(const float* proj, long long stride, int q_rank, const float* q_gain, void* cq, int kv_col,
                                          int kv_rank, const float* kv_gain, void* pages, int page_width, int rot_col, int rot,
                                          const float* cos, const float* sin, int style, int dtype, const int32_t* tok_pos,
@@ -221,19 +217,11 @@ extern "C" int rb_latent_norm_rope_store(const float* proj, long long stride, in
   if (dtype == RB_F32)
     latent_norm_store_kernel<float><<<n_tokens, 256, 0, s>>>(proj, (size_t)stride, q_rank, q_gain, (float*)cq, kv_col, kv_rank,
                                                              kv_gain, (float*)pages, page_width, tok_pos, tok_seq, block_table,
-                                                             bt_stride, eps);
+                                                             bt_stride, eps, rot_col, rot, cos, sin, style);
   else
     latent_norm_store_kernel<bf16_t><<<n_tokens, 256, 0, s>>>(proj, (size_t)stride, q_rank, q_gain, (bf16_t*)cq, kv_col, kv_rank,
                                                               kv_gain, (bf16_t*)pages, page_width, tok_pos, tok_seq, block_table,
-                                                              bt_stride, eps);
-  if (kv_rank > 0 && page_width > kv_rank) {
-    if (dtype == RB_F32)
-      latent_rope_store_kernel<float><<<n_tokens, 64, 0, s>>>(proj, (size_t)stride, kv_rank, page_width, rot_col, rot, cos, sin,
-                                                              style, (float*)pages, tok_pos, tok_seq, block_table, bt_stride);
-    else
-      latent_rope_store_kernel<bf16_t><<<n_tokens, 64, 0, s>>>(proj, (size_t)stride, kv_rank, page_width, rot_col, rot, cos, sin,
-                                                               style, (bf16_t*)pages, tok_pos, tok_seq, block_table, bt_stride);
-  }
+                                                              bt_stride, eps, rot_col, rot, cos, sin, style);
   RB_LAUNCH_CHECK();
   return 0;
 }

@@ -105,7 +105,7 @@ class KernelTimes:
         return "\n".join(lines)
 
 
-TIMED_OPS = ("outnorm_residual", "clamped_glu", "tanh_cast", "attention_opts", "norm_rope_store", "sigmoid_gate", "shift_mix", "time_mix_recurrence", "latent_norm_rope_store", "rope_heads_part", "heads_linear_part", "route_choose", "experts_combine", "embed_scaled_pos", "scale", "bias_norm_store", "attention_mixed", "attention_mixed_bf16", "recurrence_prep", "linear_recurrence", "layernorm_residual", "rope_store", "head_gate", "pair_norm_mean",
+TIMED_OPS = ("short_conv_bias", "decay_exp_exp", "gated_rmsnorm_heads", "outnorm_residual", "clamped_glu", "tanh_cast", "attention_opts", "norm_rope_store", "sigmoid_gate", "shift_mix", "time_mix_recurrence", "latent_norm_rope_store", "rope_heads_part", "heads_linear_part", "route_choose", "experts_combine", "embed_scaled_pos", "scale", "bias_norm_store", "attention_mixed", "attention_mixed_bf16", "recurrence_prep", "linear_recurrence", "layernorm_residual", "rope_store", "head_gate", "pair_norm_mean",
              "route_top", "routed_experts", "pairs_sum", "embed_streams", "streams_layernorm", "streams_update", "xielu", "tanh_cap", "short_conv",
              "delta_prep", "delta_rule", "gated_rmsnorm", "latent_norm_store", "heads_linear", "attention_sinks", "embed_gather", "add_rmsnorm", "rope_kv_write", "swiglu", "gemm_generic", "gemm_bf16", "gemm_bf16_terms",
              "gemm_bf16_few", "attention_generic", "attention_prefill_bf16", "attention_decode_bf16",
@@ -431,7 +431,7 @@ class Kernels:
             raise KernelError("decode attention workspace too small")
         if sinks is not None:
             _check(sinks, "sinks", torch.float32, (n_heads,))
-        if keep_first or softcap:
+        if keep_first or softcap or n_heads // n_kv > 16:        # this entry point also runs more than 16 heads on a kv head, in groups
             self._ok(self._lib.rb_attention_decode_bf16_opts(_ptr(q), _ptr(k_pages), _ptr(v_pages), _ptr(out), _ptr(tok_pos),
                                                              _ptr(block_table), block_table.shape[1], n, n_heads, n_kv,
                                                              head_dim, float(scale), int(window or 0), int(keep_first or 0),

@@ -298,6 +298,8 @@ extern "C" int rb_pair_norm_mean(const float* a, const float* wa, const float* b
 // rb_rope_store with every query and key head first RMS-normed over its `dim` numbers with a weight of that size shared by
 // the heads (q_norm, k_norm; plain weights): x / sqrt(mean(x^2) + eps) * w, in float32, then the rotation of the head's
 // first `rot` numbers, the padding and the cache write as there.  A wave takes a head.
+#define NRS_MAX_DIM 512
+#define NRS_MAX_WAVES 16
 template <typename TC>
 __global__ void norm_rope_store_kernel(const float* __restrict__ qkv, size_t row_width, const float* __restrict__ cos_t,
                                        const float* __restrict__ sin_t, int rot, const float* __restrict__ q_norm,
@@ -305,6 +307,8 @@ __global__ void norm_rope_store_kernel(const float* __restrict__ qkv, size_t row
                                        TC* __restrict__ k_pages, TC* __restrict__ v_pages, const int32_t* __restrict__ tok_pos,
                                        const int32_t* __restrict__ tok_seq, const int32_t* __restrict__ block_table,
                                        int bt_stride, int n_heads, int n_kv, int dim, int vdim, int pad) {
+  // a wave reads its head once (whole lines), leaves the normed head in an LDS row of its own and rotates from there
+  __shared__ float stage[NRS_MAX_WAVES][NRS_MAX_DIM];
   const int t = blockIdx.x;
   const int pos = tok_pos[t];
   const int half = rot / 2;
@@ -312,6 +316,7 @@ __global__ void norm_rope_store_kernel(const float* __restrict__ qkv, size_t row
   const float* src = qkv + (size_t)t * row_width;
   const float* cr = cos_t + (size_t)pos * half;
   const float* sr = sin_t + (size_t)pos * half;
+  float* mine = stage[wave];
   size_t page_base = 0;
   if (k_pages) {
     const int page = block_table[(size_t)tok_seq[t] * bt_stride + pos / RB_PAGE];
@@ -321,24 +326,37 @@ __global__ void norm_rope_store_kernel(const float* __restrict__ qkv, size_t row
   for (int h = wave; h < n_rot_heads; h += n_waves) {
     const float* hp = src + (size_t)h * dim;
     const float* w = h < n_heads ? q_norm : k_norm;
+    float xv[NRS_MAX_DIM / RB_WAVE];
     float ss = 0.f;
-    for (int d = lane; d < dim; d += RB_WAVE) ss = fmaf(hp[d], hp[d], ss);
+#pragma unroll
+    for (int i = 0; i < NRS_MAX_DIM / RB_WAVE; ++i) {
+      const int d = lane + RB_WAVE * i;
+      xv[i] = d < dim ? hp[d] : 0.f;
+      ss = fmaf(xv[i], xv[i], ss);
+    }
     const float f = 1.0f / sqrtf(wave_sum(ss) / (float)dim + eps);
+#pragma unroll
+    for (int i = 0; i < NRS_MAX_DIM / RB_WAVE; ++i) {
+      const int d = lane + RB_WAVE * i;
+      if (d < dim) mine[d] = xv[i] * f * w[d];
+    }
+    __builtin_amdgcn_wave_barrier();          // the row is this wave's alone; a wave's LDS accesses complete in order
     TC* dst = h < n_heads ? q_out + ((size_t)t * n_heads + h) * pad
                           : k_pages + page_base + (size_t)(h - n_heads) * RB_PAGE * pad;
     for (int d = lane; d < pad; d += RB_WAVE) {
       float y = 0.f;
       if (d < half) {
         float y1;
-        rotate_pair(hp[d] * f * w[d], hp[d + half] * f * w[d + half], cr[d], sr[d], y, y1);
+        rotate_pair(mine[d], mine[d + half], cr[d], sr[d], y, y1);
       } else if (d < rot) {
         float y0;
-        rotate_pair(hp[d - half] * f * w[d - half], hp[d] * f * w[d], cr[d - half], sr[d - half], y0, y);
+        rotate_pair(mine[d - half], mine[d], cr[d - half], sr[d - half], y0, y);
       } else if (d < dim) {
-        y = hp[d] * f * w[d];
+        y = mine[d];
       }
       Num<TC>::store(dst + d, y);
     }
+    __builtin_amdgcn_wave_barrier();
   }
   if (v_pages) {
     const float* vsrc = src + (size_t)(n_heads + n_kv) * dim;
@@ -359,6 +377,7 @@ extern "C" int rb_norm_rope_store(const float* qkv, long long row_width, const f
   RB_REQUIRE(n_tokens >= 0 && n_heads > 0 && n_kv_heads >= 0 && dim > 0 && vdim > 0 && pad >= dim && pad >= vdim,
              "rb_norm_rope_store: bad sizes T=%d Hq=%d Hk=%d dim=%d vdim=%d pad=%d", n_tokens, n_heads, n_kv_heads, dim, vdim, pad);
   RB_REQUIRE(rot >= 0 && rot % 2 == 0 && rot <= dim, "rb_norm_rope_store: %d rotated numbers in a head of %d", rot, dim);
+  RB_REQUIRE(dim <= NRS_MAX_DIM, "rb_norm_rope_store: head size %d not supported (at most %d)", dim, NRS_MAX_DIM);
   RB_REQUIRE(rot == 0 || (cos != nullptr && sin != nullptr), "rb_norm_rope_store: a rotation needs its tables");
   RB_REQUIRE(q_norm != nullptr && (k_pages == nullptr || k_norm != nullptr), "rb_norm_rope_store: the norms' weights are needed");
   RB_REQUIRE((k_pages == nullptr) == (v_pages == nullptr), "rb_norm_rope_store: k and v pages go together");
@@ -368,7 +387,8 @@ extern "C" int rb_norm_rope_store(const float* qkv, long long row_width, const f
   hipStream_t s = (hipStream_t)stream;
   // a wave a head, up to 16 waves a token: a wave's heads are a chain of trips to memory
   int waves = n_heads + (k_pages ? n_kv_heads : 0);
-  waves = waves > 16 ? 16 : (waves < 4 ? 4 : waves);
+  const int most = n_tokens < 2 * rb_compute_units() ? NRS_MAX_WAVES : 8;
+  waves = waves > most ? most : (waves < 4 ? 4 : waves);
   const int threads = RB_WAVE * waves;
   if (cache_dtype == RB_F32)
     norm_rope_store_kernel<float><<<n_tokens, threads, 0, s>>>(qkv, (size_t)row_width, cos, sin, rot, q_norm, k_norm, eps, (float*)q_out,

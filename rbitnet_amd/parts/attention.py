@@ -291,7 +291,7 @@ class Attention(Part):
         attn = torch.empty((t, hq * d), dtype=self.env.dtype, device=h.device)
         window = int(self.window) if self.window is not None else 0
         fast = (self.env.dtype == torch.bfloat16 and d in _MATRIX_CORE_HEAD_DIMS and not getattr(self.env, "generic_only", False))
-        if fast and ctx.max_q_len == 1 and (hq // hk) in _DECODE_GROUPS:
+        if fast and ctx.max_q_len == 1:
             n_splits, workspace = ctx.decode_workspace(hq, d, hk)
             lib.attention_decode_bf16(q, view.k_pages, view.v_pages, attn, ctx.tok_pos, view.block_table, hq, hk, d, self.scale,
                                       window, n_splits, workspace, sinks=self.sink, keep_first=self.keep_first,

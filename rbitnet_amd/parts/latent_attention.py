@@ -40,7 +40,6 @@ DEFAULT_NAMES = {"dq": "dq", "dq_norm": "dq.norm", "uq": "uq", "dkv": "dkv", "dk
                  "sink": "sink", "o": "o", "gate": "g"}
 MAX_RANK = 512             # the attention kernel's largest head size
 _MATRIX_CORE_RANKS = (64, 128)     # latents of these sizes in bfloat16 go through the matrix-core attention kernels
-_DECODE_MAX_HEADS = 16             # query heads on one key/value head that the matrix-core decode kernel takes
 
 
 class LatentAttention(Part):
@@ -158,7 +157,7 @@ class LatentAttention(Part):
         ol = torch.empty((t, self.heads * r), dtype=dt, device=h.device)
         q3, pages = ql.view(t, self.heads, r), view.k_pages
         fast = dt == torch.bfloat16 and r in _MATRIX_CORE_RANKS and not getattr(self.env, "generic_only", False)
-        if fast and ctx.max_q_len == 1 and self.heads <= _DECODE_MAX_HEADS:
+        if fast and ctx.max_q_len == 1:      # more than 16 heads on the latent run as several groups of at most 16
             n_splits, workspace = ctx.decode_workspace(self.heads, r, 1)
             lib.attention_decode_bf16(q3, pages, pages, ol, ctx.tok_pos, view.block_table, self.heads, 1, r, self.scale, None,
                                       n_splits, workspace, sinks=self.sink)

@@ -163,6 +163,8 @@ LATENTS = [
     dict(heads=1, dim=5, rot_dim=2, vdim=7, q_rank=3, kv_rank=9, scale=0.5, rot={"base": 7.0, "dims": 2}),           # one head, odd sizes
     dict(heads=20, dim=24, rot_dim=8, vdim=8, q_rank=64, kv_rank=64, scale=0.12, rot={"base": 300.0, "dims": 8}),   # more heads than a decode group takes
     dict(heads=2, dim=64, rot_dim=64, vdim=64, q_rank=128, kv_rank=192, scale=0.08, rot={"base": 1e4, "dims": 64}),  # 256: beyond the matrix cores' sizes
+    dict(heads=32, dim=16, rot_dim=16, vdim=8, q_rank=32, kv_rank=48, scale=0.2, rot={"base": 1e3, "dims": 16}),     # 64 a token, two groups of 16 heads
+    dict(heads=20, dim=8, rot_dim=16, vdim=16, q_rank=24, kv_rank=112, scale=0.1, rot={"base": 50.0, "dims": 16}),   # 128 a token, two groups of 10
 ]
 
 
