@@ -359,6 +359,13 @@ int rb_gated_rmsnorm_heads(const float* o, const float* weight, long long weight
 // y_head_stride (the first n are written).
 int rb_heads_linear_strided(const void* x, int x_dtype, long long x_head_stride, const void* w, int w_dtype, void* y, int y_dtype,
                             long long y_head_stride, int n_tokens, int n_heads, int n, int k, void* stream);
+// rb_heads_linear_strided with two things in the same launch: a gate per head on the outputs (gate float32, rows gate_stride
+// apart, null: none: head h of token t times sigmoid(gate[t * gate_stride + h])), and (rot >= 0) the `rot` numbers at x_rot_col
+// of every head of x rotated by the token's position into y at y_rot_col >= n, with zeros behind them up to y_head_stride.
+int rb_heads_linear_more(const void* x, int x_dtype, long long x_head_stride, const void* w, int w_dtype, void* y, int y_dtype,
+                         long long y_head_stride, int n_tokens, int n_heads, int n, int k, const float* gate, long long gate_stride,
+                         int rot, int x_rot_col, int y_rot_col, const float* cos, const float* sin, int style,
+                         const int32_t* tok_pos, void* stream);
 // rb_latent_norm_store into pages [n_pages, 1, 64, page_width] with, behind the latent, the `rot` numbers at rot_col of the
 // row rotated by the token's position (style 0: 2i with 2i + 1; 1: i with i + rot / 2) and zeros up to page_width.
 int rb_latent_norm_rope_store(const float* proj, long long stride, int q_rank, const float* q_gain, void* cq, int kv_col,

@@ -91,12 +91,37 @@ extern "C" int rb_latent_norm_store(const float* proj, long long stride, int q_r
 template <typename TX, typename TW, typename TY>
 __global__ __launch_bounds__(RB_WAVE * HL_WAVES) void heads_linear_kernel(const TX* __restrict__ x, const TW* __restrict__ w,
                                                                           TY* __restrict__ y, int n_tokens, int n_heads, int n, int k,
-                                                                          size_t x_hs, size_t y_hs) {
+                                                                          size_t x_hs, size_t y_hs, const float* __restrict__ gate,
+                                                                          size_t gate_stride, int rot, int x_rot_col, int y_rot_col,
+                                                                          const float* __restrict__ cos_t,
+                                                                          const float* __restrict__ sin_t, int style,
+                                                                          const int32_t* __restrict__ tok_pos, int n_col_tiles) {
   extern __shared__ float xs[];                  // [HL_TOKENS][k], then [HL_WAVES - 1][HL_TOKENS][64] partial sums
   float* part = xs + HL_TOKENS * k;
   const int t0 = blockIdx.x * HL_TOKENS, h = blockIdx.y;
   const int lane = threadIdx.x & (RB_WAVE - 1), wave = threadIdx.x / RB_WAVE;
   const int nt = n_tokens - t0 < HL_TOKENS ? n_tokens - t0 : HL_TOKENS;
+  if ((int)blockIdx.z == n_col_tiles) {
+    // one more workgroup per (tokens, head): the `rot` numbers at x_rot_col of the head, rotated by the token's position, go to
+    // y at y_rot_col, and what lies behind them in the head of y becomes zero
+    const int half = rot / 2, tail = (int)y_hs - y_rot_col - rot, per = half + tail;
+    for (int idx = threadIdx.x; idx < nt * per; idx += blockDim.x) {
+      const int tt = idx / per, i = idx - tt * per;
+      const TX* src = x + ((size_t)(t0 + tt) * n_heads + h) * x_hs + x_rot_col;
+      TY* dst = y + ((size_t)(t0 + tt) * n_heads + h) * y_hs + y_rot_col;
+      if (i < half) {
+        const size_t at = (size_t)tok_pos[t0 + tt] * half + i;
+        const int a = style == 0 ? 2 * i : i, b = style == 0 ? 2 * i + 1 : i + half;
+        float y0, y1;
+        rotate_pair(Num<TX>::load(src + a), Num<TX>::load(src + b), cos_t[at], sin_t[at], y0, y1);
+        Num<TY>::store(dst + a, y0);
+        Num<TY>::store(dst + b, y1);
+      } else {
+        Num<TY>::store(dst + rot + (i - half), 0.f);
+      }
+    }
+    return;
+  }
   // the tokens' inputs, eight loads in flight per lane (a step of few tokens is a chain of trips to memory otherwise)
   for (int base = 0; base < HL_TOKENS * k; base += 8 * RB_WAVE * HL_WAVES) {
     float v[8];
@@ -147,16 +172,31 @@ __global__ __launch_bounds__(RB_WAVE * HL_WAVES) void heads_linear_kernel(const 
     float v = acc[tt];
 #pragma unroll
     for (int ww = 0; ww < HL_WAVES - 1; ++ww) v += part[(ww * HL_TOKENS + tt) * RB_WAVE + lane];
-    if (tt < nt) Num<TY>::store(y + ((size_t)(t0 + tt) * n_heads + h) * y_hs + col, v);
+    if (tt < nt) {
+      if (gate) v *= 1.0f / (1.0f + expf(-gate[(size_t)(t0 + tt) * gate_stride + h]));      // a gate per head on the way out
+      Num<TY>::store(y + ((size_t)(t0 + tt) * n_heads + h) * y_hs + col, v);
+    }
   }
 }
 
+struct HeadsLinearMore {      // what rides in the same launch: a gate per head on the outputs, a rotated part beside them
+  const float* gate = nullptr;
+  size_t gate_stride = 0;
+  int rot = 0, x_rot_col = 0, y_rot_col = 0, style = 0;
+  const float* cos_t = nullptr;
+  const float* sin_t = nullptr;
+  const int32_t* tok_pos = nullptr;
+  bool has_rot = false;
+};
 template <typename TX, typename TW, typename TY>
 static void launch_heads_linear(const void* x, const void* w, void* y, int n_tokens, int n_heads, int n, int k, size_t x_hs,
-                                size_t y_hs, hipStream_t s) {
-  dim3 grid((n_tokens + HL_TOKENS - 1) / HL_TOKENS, n_heads, (n + RB_WAVE - 1) / RB_WAVE);
+                                size_t y_hs, hipStream_t s, const HeadsLinearMore& m = HeadsLinearMore()) {
+  const int n_col_tiles = (n + RB_WAVE - 1) / RB_WAVE;
+  dim3 grid((n_tokens + HL_TOKENS - 1) / HL_TOKENS, n_heads, n_col_tiles + (m.has_rot ? 1 : 0));
   const size_t lds = ((size_t)HL_TOKENS * k + (size_t)(HL_WAVES - 1) * HL_TOKENS * RB_WAVE) * sizeof(float);
-  heads_linear_kernel<TX, TW, TY><<<grid, RB_WAVE * HL_WAVES, lds, s>>>((const TX*)x, (const TW*)w, (TY*)y, n_tokens, n_heads, n, k, x_hs, y_hs);
+  heads_linear_kernel<TX, TW, TY><<<grid, RB_WAVE * HL_WAVES, lds, s>>>((const TX*)x, (const TW*)w, (TY*)y, n_tokens, n_heads, n, k, x_hs,
+                                                                        y_hs, m.gate, m.gate_stride, m.rot, m.x_rot_col, m.y_rot_col,
+                                                                        m.cos_t, m.sin_t, m.style, m.tok_pos, n_col_tiles);
 }
 
 extern "C" int rb_heads_linear(const void* x, int x_dtype, const void* w, int w_dtype, void* y, int y_dtype, int n_tokens,
@@ -171,6 +211,38 @@ extern "C" int rb_heads_linear_strided(const void* x, int x_dtype, long long x_h
                                        int y_dtype, long long y_head_stride, int n_tokens, int n_heads, int n, int k, void* stream) {
   RB_RECORDED(rb_heads_linear_strided(x, x_dtype, x_head_stride, w, w_dtype, y, y_dtype, y_head_stride, n_tokens, n_heads, n, k,
                                       stream));
+  return rb_heads_linear_more(x, x_dtype, x_head_stride, w, w_dtype, y, y_dtype, y_head_stride, n_tokens, n_heads, n, k, nullptr, 0,
+                              -1, 0, 0, nullptr, nullptr, 0, nullptr, stream);
+}
+
+// The same with two things in the same launch.  gate (float32, rows gate_stride apart; null: none): head h's outputs of token t
+// are multiplied by sigmoid(gate[t * gate_stride + h]).  rot >= 0 (rot < 0: none): the `rot` numbers at x_rot_col of every head
+// of x, rotated by the token's position (cos, sin [positions, rot / 2]; style 0: 2i with 2i + 1, 1: i with i + rot / 2), go to
+// y at y_rot_col, and what lies behind them in a head of y becomes zero.
+extern "C" int rb_heads_linear_more(const void* x, int x_dtype, long long x_head_stride, const void* w, int w_dtype, void* y,
+                                    int y_dtype, long long y_head_stride, int n_tokens, int n_heads, int n, int k, const float* gate,
+                                    long long gate_stride, int rot, int x_rot_col, int y_rot_col, const float* cos, const float* sin,
+                                    int style, const int32_t* tok_pos, void* stream) {
+  RB_RECORDED(rb_heads_linear_more(x, x_dtype, x_head_stride, w, w_dtype, y, y_dtype, y_head_stride, n_tokens, n_heads, n, k, gate,
+                                   gate_stride, rot, x_rot_col, y_rot_col, cos, sin, style, tok_pos, stream));
+  HeadsLinearMore more;
+  more.gate = gate;
+  more.gate_stride = (size_t)gate_stride;
+  RB_REQUIRE(gate == nullptr || gate_stride >= n_heads, "rb_heads_linear: the gate's rows are shorter than the heads");
+  if (rot >= 0) {
+    RB_REQUIRE(rot % 2 == 0 && x_rot_col >= 0 && y_rot_col >= n && x_head_stride >= (long long)x_rot_col + rot &&
+                   y_head_stride >= (long long)y_rot_col + rot,
+               "rb_heads_linear: the rotated part lies outside a head, or over the product's outputs");
+    RB_REQUIRE(rot == 0 || (cos && sin && tok_pos && (style == 0 || style == 1)), "rb_heads_linear: a rotation needs its tables");
+    more.has_rot = y_head_stride > y_rot_col;
+    more.rot = rot;
+    more.x_rot_col = x_rot_col;
+    more.y_rot_col = y_rot_col;
+    more.style = style;
+    more.cos_t = cos;
+    more.sin_t = sin;
+    more.tok_pos = tok_pos;
+  }
   RB_REQUIRE(n_tokens >= 0 && n_heads > 0 && n_heads <= 65535 && n > 0 && n <= 65535 * 64 && k > 0, "rb_heads_linear: bad sizes");
   RB_REQUIRE(k <= 768, "rb_heads_linear: inner size %d not supported (at most 768)", k);
   RB_REQUIRE(x_head_stride >= k && y_head_stride >= n, "rb_heads_linear: a head's stride is shorter than the head");
@@ -179,11 +251,11 @@ extern "C" int rb_heads_linear_strided(const void* x, int x_dtype, long long x_h
   const size_t xs = (size_t)x_head_stride, ys = (size_t)y_head_stride;
   const int key = x_dtype * 4 + w_dtype * 2 + y_dtype;
   switch (key) {
-    case 0: launch_heads_linear<float, float, float>(x, w, y, n_tokens, n_heads, n, k, xs, ys, s); break;
-    case 3: launch_heads_linear<float, bf16_t, bf16_t>(x, w, y, n_tokens, n_heads, n, k, xs, ys, s); break;
-    case 6: launch_heads_linear<bf16_t, bf16_t, float>(x, w, y, n_tokens, n_heads, n, k, xs, ys, s); break;
-    case 7: launch_heads_linear<bf16_t, bf16_t, bf16_t>(x, w, y, n_tokens, n_heads, n, k, xs, ys, s); break;
-    case 2: launch_heads_linear<float, bf16_t, float>(x, w, y, n_tokens, n_heads, n, k, xs, ys, s); break;
+    case 0: launch_heads_linear<float, float, float>(x, w, y, n_tokens, n_heads, n, k, xs, ys, s, more); break;
+    case 3: launch_heads_linear<float, bf16_t, bf16_t>(x, w, y, n_tokens, n_heads, n, k, xs, ys, s, more); break;
+    case 6: launch_heads_linear<bf16_t, bf16_t, float>(x, w, y, n_tokens, n_heads, n, k, xs, ys, s, more); break;
+    case 7: launch_heads_linear<bf16_t, bf16_t, bf16_t>(x, w, y, n_tokens, n_heads, n, k, xs, ys, s, more); break;
+    case 2: launch_heads_linear<float, bf16_t, float>(x, w, y, n_tokens, n_heads, n, k, xs, ys, s, more); break;
     default: RB_REQUIRE(false, "rb_heads_linear: this combination of types is not built (x %d, w %d, y %d)", x_dtype, w_dtype, y_dtype);
   }
   RB_LAUNCH_CHECK();

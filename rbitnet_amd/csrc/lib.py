@@ -193,6 +193,7 @@ class Kernels:
             "rb_short_conv_bias": [_P, _L, _P, _P, _I, _P, _P, _P, _P, _P, _P, _L, _I, _I, _I, _I, _I, _I, _P],
             "rb_linear_recurrence_bonus": [_P, _P, _L, _P, _L, _P, _L, _I, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P],
             "rb_gated_rmsnorm_heads": [_P, _P, _L, _P, _L, _I, _F, _P, _I, _I, _I, _I, _P],
+            "rb_heads_linear_more": [_P, _I, _L, _P, _I, _P, _I, _L, _I, _I, _I, _I, _P, _L, _I, _I, _I, _P, _P, _I, _P, _P],
             "rb_heads_linear_strided": [_P, _I, _L, _P, _I, _P, _I, _L, _I, _I, _I, _I, _P],
             "rb_latent_norm_rope_store": [_P, _L, _I, _P, _P, _I, _I, _P, _P, _I, _I, _I, _P, _P, _I, _I, _P, _P, _P, _I, _F, _I, _P],
             "rb_rope_heads_part": [_P, _L, _I, _I, _P, _P, _I, _P, _I, _L, _I, _P, _I, _I, _P],
@@ -1192,8 +1193,11 @@ class Kernels:
         self._ok(self._lib.rb_gated_rmsnorm_heads(_ptr(o), _ptr(weight), vdim, _ptr(gate), n_heads * vdim, int(act), float(eps),
                                                   _ptr(out), dtype_code(out.dtype), n, n_heads, vdim, self._stream()))
 
-    def heads_linear_part(self, x: torch.Tensor, x_head: int, w: torch.Tensor, y: torch.Tensor, y_head: int) -> None:
-        """y[t, h, :N] = w[h]^T x[t, h, :K] with w [H, K, N]; a head of x takes x_head numbers, a head of y y_head."""
+    def heads_linear_part(self, x: torch.Tensor, x_head: int, w: torch.Tensor, y: torch.Tensor, y_head: int,
+                          gate: Optional[torch.Tensor] = None, gate_col: int = 0, rope=None) -> None:
+        """y[t, h, :N] = w[h]^T x[t, h, :K] with w [H, K, N]; a head of x takes x_head numbers, a head of y y_head.
+        gate [T, >= gate_col + H] float32: head h's outputs times sigmoid(gate[:, gate_col + h]).  rope = (x_col, rot, cos, sin,
+        style, y_col, tok_pos): the rot numbers at x_col of every head of x, rotated, go to y at y_col, zeros behind them."""
         h, k, n_out = w.shape
         n = x.shape[0]
         _check(x, "x", None, (n, h * x_head))
@@ -1201,8 +1205,27 @@ class Kernels:
         _check(y, "y", None, (n, h * y_head))
         if x_head < k or y_head < n_out:
             raise KernelError("heads_linear_part: a head is shorter than the product's sizes")
-        self._ok(self._lib.rb_heads_linear_strided(_ptr(x), dtype_code(x.dtype), x_head, _ptr(w), dtype_code(w.dtype), _ptr(y),
-                                                   dtype_code(y.dtype), y_head, n, h, n_out, k, self._stream()))
+        g_ptr, g_stride = None, 0
+        if gate is not None:
+            _check(gate, "gate", torch.float32)
+            if gate.shape[0] != n or gate_col < 0 or gate_col + h > gate.shape[1]:
+                raise KernelError("heads_linear_part: the gate's columns lie outside the rows")
+            g_ptr, g_stride = gate.data_ptr() + 4 * gate_col, gate.shape[1]
+        rot, x_col, y_col, cos, sin, style, tok_pos = -1, 0, 0, None, None, 0, None
+        if rope is not None:
+            x_col, rot, cos, sin, style, y_col, tok_pos = rope
+            if x.dtype != torch.float32 or x_col + rot > x_head or y_col + rot > y_head or y_col < n_out:
+                raise KernelError("heads_linear_part: the rotated part lies outside a head, or x is not float32")
+            _check(tok_pos, "tok_pos", torch.int32, (n,))
+            if rot:
+                _check(cos, "cos", torch.float32)
+                _check(sin, "sin", torch.float32, cos.shape)
+                if cos.shape[1] != rot // 2:
+                    raise KernelError("angle table width mismatch")
+        self._ok(self._lib.rb_heads_linear_more(_ptr(x), dtype_code(x.dtype), x_head, _ptr(w), dtype_code(w.dtype), _ptr(y),
+                                                dtype_code(y.dtype), y_head, n, h, n_out, k, g_ptr, g_stride, int(rot), int(x_col),
+                                                int(y_col), _ptr(cos) if rot > 0 else None, _ptr(sin) if rot > 0 else None, int(style),
+                                                _ptr(tok_pos), self._stream()))
 
     def latent_norm_rope_store(self, proj: torch.Tensor, q_rank: int, q_gain, cq, kv_rank: int, kv_gain, pages, rot: int, cos, sin,
                                style: int, ctx, block_table, eps: float, dtype: torch.dtype) -> None:

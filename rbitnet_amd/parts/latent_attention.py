@@ -149,9 +149,8 @@ class LatentAttention(Part):
         ql = torch.empty((t, self.heads * r), dtype=dt, device=h.device)
         if self.rot:
             # the queries in the cache's layout: the unrotated part in the latent's space, then the rotated part, then zeros
-            lib.heads_linear_part(q, self.dim + self.rot, self.w_uk, ql, r)
-            lib.rope_heads_part(q, self.dim + self.rot, self.dim, self.rot, cos, sin, style, ql, r, self.kv_rank, ctx.tok_pos,
-                                self.heads)
+            lib.heads_linear_part(q, self.dim + self.rot, self.w_uk, ql, r,
+                                  rope=(self.dim, self.rot, cos, sin, style, self.kv_rank, ctx.tok_pos))
         else:
             lib.heads_linear(q, self.w_uk, ql)                                # the queries in the latent's space
         ol = torch.empty((t, self.heads * r), dtype=dt, device=h.device)
@@ -168,12 +167,8 @@ class LatentAttention(Part):
             lib.attention_sinks(q3, pages, pages, ol, ctx.tok_pos, ctx.tok_seq, view.block_table, self.heads, 1, r,
                                 self.scale, None, self.sink)
         o = torch.empty((t, self.heads * self.vdim), dtype=dt, device=h.device)
-        if self.rot:
-            lib.heads_linear_part(ol, r, self.w_uv, o, self.vdim)             # the latent's part of every head's sum
-        else:
-            lib.heads_linear(ol, self.w_uv, o)
-        if self.has_gate:
-            lib.head_gate(o, down, self.gate_col, self.heads, self.vdim)
+        # the latent's part of every head's sum through the head's value matrix, the head's gate on the way out
+        lib.heads_linear_part(ol, r, self.w_uv, o, self.vdim, gate=down if self.has_gate else None, gate_col=self.gate_col)
         return linear(lib, o, self.w_o, torch.float32)
 
 
