@@ -37,7 +37,7 @@ GATE_ALPHA = 1.702             # the feed-forward's gate is g * sigmoid(1.702 g)
 
 def _rot(m: Dict[str, Any], where: str, limit: int) -> Dict[str, Any]:
     rot = _obj(m, "rot", where)
-    dims = _int(rot, "dims", f"{where} rot")
+    dims = _int(rot, "dims", f"{where} rot", zero_ok=True)
     if not _float(rot, "base", f"{where} rot") > 0:
         raise ConfigError(f"{where} rot: base must be positive")
     if dims % 2 != 0 or dims > limit:
@@ -93,10 +93,11 @@ class MeneraxConfig:
                                   f"{layer.get('type') if isinstance(layer, dict) else layer!r}")
             m = _obj(layer, "mixer", where)
             if layer["type"] == "latent_attention":
-                for key in ("heads", "dim", "rot_dim", "vdim", "q_rank", "kv_rank"):
+                for key in ("heads", "dim", "vdim", "q_rank", "kv_rank"):
                     _int(m, key, where)
+                _int(m, "rot_dim", where, zero_ok=True)
                 _float(m, "scale", where)
-                if _rot(m, where, m["rot_dim"])["dims"] != m["rot_dim"]:
+                if (m["rot_dim"] or m.get("rot") is not None) and _rot(m, where, m["rot_dim"])["dims"] != m["rot_dim"]:
                     raise ConfigError(f"{where}: the rotated part has rot_dim = {m['rot_dim']} numbers and all of them are rotated, "
                                       f"found rot.dims = {m['rot']['dims']}")
             else:
@@ -162,8 +163,8 @@ class MeneraxConfig:
     def _latent(self, m: Dict[str, Any]) -> PartSpec:
         return PartSpec("latent_attention", {
             "heads": m["heads"], "dim": m["dim"], "vdim": m["vdim"], "q_rank": m["q_rank"], "kv_rank": m["kv_rank"],
-            "scale": m["scale"], "eps": self.norm_eps, "rot_dim": m["rot_dim"], "position": self._position(m["rot"], "interleaved"),
-            "sink": False, "head_gate": True})
+            "scale": m["scale"], "eps": self.norm_eps, "rot_dim": m["rot_dim"],
+            "position": self._position(m["rot"], "interleaved") if m["rot_dim"] else None, "sink": False, "head_gate": True})
 
     def _left(self, m: Dict[str, Any]) -> PartSpec:
         mask = m.get("mask")

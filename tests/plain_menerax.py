@@ -116,7 +116,7 @@ def latent_attention(h, w: Dict[str, torch.Tensor], p: Dict, eps: float):
     rotated part that all heads share."""
     t_len = h.shape[0]
     heads, d, r, dv, rank = p["heads"], p["dim"], p["rot_dim"], p["vdim"], p["kv_rank"]
-    f = frequencies(p["rot"]["dims"], p["rot"]["base"], p["rot"].get("scaling"))
+    f = frequencies(p["rot"]["dims"], p["rot"]["base"], p["rot"].get("scaling")) if r else torch.zeros(0, dtype=F64)
     cq = norm_plain(h @ w["dq"].T, w["dq.norm"], eps)
     q = (cq @ w["uq"].T).view(t_len, heads, d + r)
     q_plain, q_rot = q[..., :d], rotate(q[..., d:], f, "pairs")

@@ -559,6 +559,103 @@ def test_long_decoding_and_greedy_generation_through_the_engine(name, dtype):
     assert eng.stats["decode_tokens"] > 0 and eng.model.graph_safe and eng.model.plan_safe
 
 
+def _random_config(rng):
+    """A model whose every size, constant, layer order and shared layer is drawn: what no hand-made model thought of."""
+    def latent():
+        rot = rng.choice([0, 2, 4, 8, 16, 32, 64])
+        out = dict(heads=rng.choice([1, 2, 3, 4, 8, 16, 24, 32]), dim=rng.choice([8, 16, 32, 64, 128]), rot_dim=rot, vdim=rng.choice([8, 16, 32, 64]),
+                   q_rank=rng.choice([16, 24, 64, 128]), kv_rank=rng.choice([8, 24, 32, 48, 64, 96, 112, 128]), scale=rng.choice([0.05, 0.125, 0.2]))
+        if rot:
+            out["rot"] = {"base": rng.choice([100.0, 1e4, 5e5]), "dims": rot}
+        return out
+
+    def parallel():
+        dim, kvh, group = rng.choice([8, 16, 32, 64, 128]), rng.choice([1, 2, 4]), rng.choice([1, 2, 3, 4, 8, 20])
+        dims = rng.choice([0, 2, dim // 2, dim])
+        rot = {"base": rng.choice([1e4, 5e5]), "dims": dims - dims % 2}
+        if rot["dims"] and rng.random() < 0.5:
+            rot["scaling"] = {"factor": rng.choice([2.0, 8.0]), "low": 1.0, "high": rng.choice([2.0, 4.0]), "original": rng.choice([16, 64, 2048])}
+        left = dict(heads=kvh * group, kv_heads=kvh, dim=dim, vdim=rng.choice([8, 16, 48, 64, 128]), conv=rng.choice([1, 2, 3, 4, 7]), rot=rot,
+                    scale=rng.choice([0.1, 0.125, 0.3]))
+        if rng.random() < 0.8:
+            left["softcap"] = rng.choice([5.0, 30.0, 50.0])
+        if rng.random() < 0.85:
+            left["mask"] = {"size": rng.choice([1, 7, 40, 64, 100, 128, 200]), "keep_first": rng.choice([0, 1, 4, 20, 64, 70, 130])}
+        right = dict(heads=rng.choice([1, 2, 6, 8]), dim=rng.choice([8, 16, 32, 64]), decay_rank=rng.choice([1, 4, 16, 24]))
+        return {"left": left, "right": right, "left_scale": rng.choice([0.6, 1.0, 1.5]), "right_scale": rng.choice([0.4, 1.1])}
+
+    layers = []
+    for _ in range(rng.choice([2, 3, 4])):
+        kind = rng.choice(["latent_attention", "parallel"])
+        mlp = None if rng.random() < 0.2 else {"kind": "dense", "ff": rng.choice([16, 40, 64, 96, 256]), "limit": rng.choice([0.5, 2.0, 7.0])}
+        layers.append({"type": kind, "mixer": latent() if kind == "latent_attention" else parallel(), "mlp": mlp})
+    for _ in range(rng.choice([0, 1, 2])):               # layers that run another layer's weights, anywhere behind it
+        owners = [i for i, l in enumerate(layers) if "weights_of" not in l]
+        j = rng.choice(owners)
+        at = rng.randrange(j + 1, len(layers) + 1)
+        for l in layers:                                  # the layers behind the new one move on by one
+            if l.get("weights_of") is not None and l["weights_of"] >= at:
+                l["weights_of"] += 1
+        layers.insert(at, dict(copy.deepcopy({k: v for k, v in layers[j].items() if k != "weights_of"}), weights_of=j))
+    return {"architecture": "Menerax", "vocab": rng.choice([37, 96, 300]), "width": rng.choice([32, 48, 64, 96, 128, 160, 256]),
+            "norm": {"eps": rng.choice([1e-5, 1e-6])}, "layers": layers}
+
+
+@pytest.mark.parametrize("seed", [16, 17, 19, 27, 29, 38])
+def test_models_drawn_at_random_whole_in_pieces_decoded_and_batched(seed, tmp_path):
+    import random
+    import rbitnet_amd
+    from rbitnet_amd.weights.safetensors_io import save_file
+    cfg = _random_config(random.Random(seed))
+    tensors = P.random_menerax_tensors(cfg, seed)
+    oracle = P.PlainMenerax(copy.deepcopy(cfg), tensors)
+    stored = copy.deepcopy(cfg)
+    for layer in stored["layers"]:
+        if layer["type"] == "parallel":
+            layer["mixer"]["right"].pop("decay_rank")
+    with open(tmp_path / "config.json", "w") as f:
+        json.dump(stored, f)
+    save_file(str(tmp_path / "model.safetensors"), [(k, v.to(torch.bfloat16)) for k, v in tensors.items()])
+    g = torch.Generator().manual_seed(seed)
+    seqs = [torch.randint(0, cfg["vocab"], (n,), generator=g).tolist() for n in (210, 75, 9)]
+    want = [oracle.logits(s) for s in seqs]
+
+    def rows(got, ref):
+        ref = ref.double().cpu()
+        return ((got.double().cpu() - ref) ** 2).mean(-1).sqrt() / ref.abs().max()
+
+    for dtype in ("float32", "bfloat16"):
+        eng = rbitnet_amd.Engine.load_path(str(tmp_path), dtype=dtype, max_seq_len=512, max_tokens=64 * 12, max_batch=4)
+        slot = eng.alloc_slot()
+        whole = eng.step([(slot, seqs[0])], "all")
+        eng.free_slot(slot)
+        slot, parts, at = eng.alloc_slot(), [], 0
+        for n in [3, 61, 2, 64, 40] + [1] * 40:
+            parts.append(eng.step([(slot, seqs[0][at:at + n])], "all"))
+            at += n
+        eng.free_slot(slot)
+        slots, heads = [eng.alloc_slot() for _ in seqs], [180, 60, 1]
+        logits = eng.step([(sl, q[:h]) for sl, q, h in zip(slots, seqs, heads)], "all")
+        got = [[logits[sum(heads[:i]):sum(heads[:i + 1])]] for i in range(3)]
+        at, live = list(heads), [0, 1, 2]
+        while live:
+            logits = eng.step([(slots[i], [seqs[i][at[i]]]) for i in live], "last")
+            for r, i in enumerate(live):
+                got[i].append(logits[r:r + 1])
+                at[i] += 1
+            for i in [i for i in live if at[i] >= len(seqs[i])]:
+                eng.free_slot(slots[i])
+                live.remove(i)
+        eng.cache.check()
+        errs = [rows(whole, want[0]), rows(torch.cat(parts), want[0])] + [rows(torch.cat(got[i]), want[i]) for i in range(3)]
+        for e in errs:
+            if dtype == "float32":
+                assert float(e.max()) < 5e-5, (seed, dtype)
+            else:
+                assert float(e.median()) < 4e-2 and float((e > 1.2e-1).double().mean()) <= 0.1, (seed, dtype)
+        del eng
+
+
 def test_replay_and_command_line_on_a_model_of_this_design(tmp_path, capsys):
     import numpy as np
     from rbitnet_amd import cli
