@@ -383,18 +383,18 @@ def menerax_config(width: int, layers: int, heads: int, kv_heads: int, ff: int, 
     latent = {"heads": heads, "dim": 64, "rot_dim": 32, "vdim": 64, "q_rank": max(256, width * 3 // 8), "kv_rank": 96, "scale": 96 ** -0.5,
               "rot": {"base": 10000.0, "dims": 32}}
     left = {"heads": heads * 64 // head, "kv_heads": max(1, kv_heads * 64 // head), "dim": head, "vdim": head, "conv": 4,
-            "rot": {"base": 500000.0, "dims": head // 2, "scaling": {"factor": 8.0, "low": 1.0, "high": 4.0, "original": 8192}},
-            "scale": head ** -0.5, "softcap": 30.0, "mask": {"size": window, "keep_first": keep_first}}
+            "rot": {"base": 1000000.0, "dims": head // 2, "scaling": {"factor": 4.0, "low": 1.0, "high": 2.0, "original": 4096}},
+            "scale": head ** -0.5, "softcap": 50.0, "mask": {"size": window, "keep_first": keep_first}}
     right = {"heads": max(1, width // 128), "dim": 64, "decay_rank": 64}
     mlp = {"kind": "dense", "ff": ff, "limit": 7.0}
     out = []
     for i in range(layers):
         if i % 4 == 2:
-            out.append({"type": "parallel", "mixer": {"left": dict(left), "right": dict(right), "left_scale": 0.6, "right_scale": 1.1},
+            out.append({"type": "parallel", "mixer": {"left": dict(left), "right": dict(right), "left_scale": 0.5, "right_scale": 1.0},
                         "mlp": dict(mlp)})
         else:
             out.append({"type": "latent_attention", "mixer": dict(latent), "mlp": dict(mlp)})
-    return {"architecture": "Menerax", "vocab": vocab, "width": width, "norm": {"eps": 1e-6}, "layers": out}
+    return {"architecture": "Menerax", "vocab": vocab, "width": width, "norm": {"eps": 1e-5}, "layers": out}
 
 
 # size -> (the design's configuration, then the shapes beside it: the Llama shape of equal width, depth and feed-forward

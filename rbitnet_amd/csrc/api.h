@@ -372,12 +372,6 @@ int rb_latent_norm_rope_store(const float* proj, long long stride, int q_rank, c
                               int kv_rank, const float* kv_gain, void* pages, int page_width, int rot_col, int rot, const float* cos,
                               const float* sin, int style, int dtype, const int32_t* tok_pos, const int32_t* tok_seq,
                               const int32_t* block_table, int bt_stride, float eps, int n_tokens, void* stream);
-// Of every head of x [T, H, x_head_stride] float32 the `rot` numbers at x_col, rotated by the token's position, go to
-// y [T, H, y_head_stride] at y_col; what lies behind them in a head of y becomes zero.
-int rb_rope_heads_part(const float* x, long long x_head_stride, int x_col, int rot, const float* cos, const float* sin, int style,
-                       void* y, int y_dtype, long long y_head_stride, int y_col, const int32_t* tok_pos, int n_tokens, int n_heads,
-                       void* stream);
-
 // tokens[r] = argmax of logits[r, :] (NaN counts as -inf, lowest index among equals), or, where
 // temperature[r] > 0, the first index whose running sum of exp(z/T - max) reaches u[r] times the total.
 // workspace: rb_sample_workspace_bytes(n_rows, vocab) bytes, 8-byte aligned, contents do not matter.

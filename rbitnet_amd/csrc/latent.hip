@@ -297,55 +297,3 @@ extern "C" int rb_latent_norm_rope_store(const float* proj, long long stride, in
   RB_LAUNCH_CHECK();
   return 0;
 }
-
-// The queries' side of the same: of every head of x [T, H, x_head_stride] float32 the `rot` numbers at x_col are rotated by the
-// token's position and written to y [T, H, y_head_stride] at y_col; what lies behind them up to y_head_stride becomes zero.
-template <typename TC>
-__global__ void rope_heads_part_kernel(const float* __restrict__ x, size_t x_hs, int x_col, int rot, const float* __restrict__ cos_t,
-                                       const float* __restrict__ sin_t, int style, TC* __restrict__ y, size_t y_hs, int y_col,
-                                       const int32_t* __restrict__ tok_pos, int n_heads) {
-  const int t = blockIdx.x;
-  const int pos = tok_pos[t];
-  const int half = rot / 2;
-  const float* cr = cos_t + (size_t)pos * half;
-  const float* sr = sin_t + (size_t)pos * half;
-  const int tail = (int)y_hs - y_col - rot;
-  const int per_head = half + tail;
-  for (int idx = threadIdx.x; idx < n_heads * per_head; idx += blockDim.x) {
-    const int h = idx / per_head, i = idx - h * per_head;
-    const float* src = x + ((size_t)t * n_heads + h) * x_hs + x_col;
-    TC* dst = y + ((size_t)t * n_heads + h) * y_hs + y_col;
-    if (i < half) {
-      const int a = style == 0 ? 2 * i : i, b = style == 0 ? 2 * i + 1 : i + half;
-      float y0, y1;
-      rotate_pair(src[a], src[b], cr[i], sr[i], y0, y1);
-      Num<TC>::store(dst + a, y0);
-      Num<TC>::store(dst + b, y1);
-    } else {
-      Num<TC>::store(dst + rot + (i - half), 0.f);
-    }
-  }
-}
-
-extern "C" int rb_rope_heads_part(const float* x, long long x_head_stride, int x_col, int rot, const float* cos, const float* sin,
-                                  int style, void* y, int y_dtype, long long y_head_stride, int y_col, const int32_t* tok_pos,
-                                  int n_tokens, int n_heads, void* stream) {
-  RB_RECORDED(rb_rope_heads_part(x, x_head_stride, x_col, rot, cos, sin, style, y, y_dtype, y_head_stride, y_col, tok_pos, n_tokens,
-                                 n_heads, stream));
-  RB_REQUIRE(n_tokens >= 0 && n_heads > 0 && rot >= 0 && rot % 2 == 0 && x_col >= 0 && y_col >= 0, "rb_rope_heads_part: bad sizes");
-  RB_REQUIRE(x_head_stride >= (long long)x_col + rot && y_head_stride >= (long long)y_col + rot,
-             "rb_rope_heads_part: the rotated part lies outside a head");
-  RB_REQUIRE(rot == 0 || (cos && sin && (style == 0 || style == 1)), "rb_rope_heads_part: a rotation needs its tables");
-  if (n_tokens == 0 || y_head_stride == y_col) return 0;
-  hipStream_t s = (hipStream_t)stream;
-  if (y_dtype == RB_F32)
-    rope_heads_part_kernel<float><<<n_tokens, 256, 0, s>>>(x, (size_t)x_head_stride, x_col, rot, cos, sin, style, (float*)y,
-                                                           (size_t)y_head_stride, y_col, tok_pos, n_heads);
-  else if (y_dtype == RB_BF16)
-    rope_heads_part_kernel<bf16_t><<<n_tokens, 256, 0, s>>>(x, (size_t)x_head_stride, x_col, rot, cos, sin, style, (bf16_t*)y,
-                                                            (size_t)y_head_stride, y_col, tok_pos, n_heads);
-  else
-    RB_REQUIRE(false, "rb_rope_heads_part: unknown dtype %d", y_dtype);
-  RB_LAUNCH_CHECK();
-  return 0;
-}

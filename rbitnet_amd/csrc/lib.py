@@ -105,7 +105,7 @@ class KernelTimes:
         return "\n".join(lines)
 
 
-TIMED_OPS = ("short_conv_bias", "decay_exp_exp", "gated_rmsnorm_heads", "outnorm_residual", "clamped_glu", "tanh_cast", "attention_opts", "norm_rope_store", "sigmoid_gate", "shift_mix", "time_mix_recurrence", "latent_norm_rope_store", "rope_heads_part", "heads_linear_part", "route_choose", "experts_combine", "embed_scaled_pos", "scale", "bias_norm_store", "attention_mixed", "attention_mixed_bf16", "recurrence_prep", "linear_recurrence", "layernorm_residual", "rope_store", "head_gate", "pair_norm_mean",
+TIMED_OPS = ("short_conv_bias", "decay_exp_exp", "gated_rmsnorm_heads", "outnorm_residual", "clamped_glu", "tanh_cast", "attention_opts", "norm_rope_store", "sigmoid_gate", "shift_mix", "time_mix_recurrence", "latent_norm_rope_store", "heads_linear_part", "route_choose", "experts_combine", "embed_scaled_pos", "scale", "bias_norm_store", "attention_mixed", "attention_mixed_bf16", "recurrence_prep", "linear_recurrence", "layernorm_residual", "rope_store", "head_gate", "pair_norm_mean",
              "route_top", "routed_experts", "pairs_sum", "embed_streams", "streams_layernorm", "streams_update", "xielu", "tanh_cap", "short_conv",
              "delta_prep", "delta_rule", "gated_rmsnorm", "latent_norm_store", "heads_linear", "attention_sinks", "embed_gather", "add_rmsnorm", "rope_kv_write", "swiglu", "gemm_generic", "gemm_bf16", "gemm_bf16_terms",
              "gemm_bf16_few", "attention_generic", "attention_prefill_bf16", "attention_decode_bf16",
@@ -196,7 +196,6 @@ class Kernels:
             "rb_heads_linear_more": [_P, _I, _L, _P, _I, _P, _I, _L, _I, _I, _I, _I, _P, _L, _I, _I, _I, _P, _P, _I, _P, _P],
             "rb_heads_linear_strided": [_P, _I, _L, _P, _I, _P, _I, _L, _I, _I, _I, _I, _P],
             "rb_latent_norm_rope_store": [_P, _L, _I, _P, _P, _I, _I, _P, _P, _I, _I, _I, _P, _P, _I, _I, _P, _P, _P, _I, _F, _I, _P],
-            "rb_rope_heads_part": [_P, _L, _I, _I, _P, _P, _I, _P, _I, _L, _I, _P, _I, _I, _P],
             "rb_attention_mixed": [_P, _P, _P, _P, _I, _P, _P, _P, _I, _I, _I, _I, _I, _F, _P, _I, _I, _P],
             "rb_attention_mixed_bf16": [_P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _P, _I, _I, _I, _P, _P],
         }
@@ -1257,24 +1256,6 @@ class Kernels:
                                                      dtype_code(dtype), _ptr(ctx.tok_pos), _ptr(ctx.tok_seq),
                                                      _ptr(block_table) if has_kv else None, block_table.shape[1] if has_kv else 0,
                                                      float(eps), n, self._stream()))
-
-    def rope_heads_part(self, x: torch.Tensor, x_head: int, x_col: int, rot: int, cos, sin, style: int, y: torch.Tensor, y_head: int,
-                        y_col: int, tok_pos, n_heads: int) -> None:
-        """The `rot` numbers at x_col of every head of x [T, H * x_head] float32, rotated, to y [T, H * y_head] at y_col; zeros behind."""
-        n = x.shape[0]
-        _check(x, "x", torch.float32, (n, n_heads * x_head))
-        _check(y, "y", None, (n, n_heads * y_head))
-        _check(tok_pos, "tok_pos", torch.int32, (n,))
-        if x_col + rot > x_head or y_col + rot > y_head:
-            raise KernelError("rope_heads_part: the rotated part lies outside a head")
-        if rot:
-            _check(cos, "cos", torch.float32)
-            _check(sin, "sin", torch.float32, cos.shape)
-            if cos.shape[1] != rot // 2:
-                raise KernelError("angle table width mismatch")
-        self._ok(self._lib.rb_rope_heads_part(_ptr(x), x_head, x_col, rot, _ptr(cos) if rot else None, _ptr(sin) if rot else None,
-                                              int(style), _ptr(y), dtype_code(y.dtype), y_head, y_col, _ptr(tok_pos), n, n_heads,
-                                              self._stream()))
 
     # ------------------------------------------------------------------ recorded steps
     def plan_begin(self) -> int:

@@ -126,7 +126,7 @@ def test_the_norm_on_a_sublayers_output_with_the_residual_sum(lib):
         part = build_part("norm", PartSpec("rmsnorm", {"size": e, "eps": 1e-4, "one_plus": True, "names": {"weight": ""}}),
                           _env(lib, e, dtype))
         part.load({"": w.float().to(DEV)})
-        for second, sa, sb in ((None, 1.0, 0.0), (b, 0.6, 1.1)):
+        for second, sa, sb in ((None, 1.0, 0.0), (b, 0.7, 1.3)):
             y = sa * a + (sb * second if second is not None else 0)
             want = x + P.norm_around_zero(y, w, 1e-4)
             xd = x.float().to(DEV)
@@ -214,10 +214,10 @@ def _left(heads, kv_heads, dim, vdim, conv, dims, base, scale, softcap=None, mas
 
 
 LEFTS = [
-    _left(4, 2, 16, 24, 3, 8, 100.0, 0.3, softcap=5.0, mask={"size": 40, "keep_first": 20}),
+    _left(4, 2, 16, 24, 3, 8, 100.0, 0.3, softcap=5.0, mask={"size": 36, "keep_first": 12}),
     _left(3, 3, 24, 8, 1, 24, 5000.0, 0.2, mask={"size": 70, "keep_first": 0}),                              # one tap, nothing kept
-    _left(8, 2, 64, 64, 4, 64, 1e4, 0.125, softcap=30.0, mask={"size": 64, "keep_first": 64},
-          scaling={"factor": 8.0, "low": 1.0, "high": 4.0, "original": 64}),                                  # the matrix cores' sizes
+    _left(8, 2, 64, 64, 4, 64, 1e4, 0.11, softcap=20.0, mask={"size": 64, "keep_first": 64},
+          scaling={"factor": 4.0, "low": 1.0, "high": 2.0, "original": 64}),                                  # the matrix cores' sizes
     _left(6, 3, 64, 128, 2, 32, 5e5, 0.1, softcap=2.0, mask={"size": 129, "keep_first": 65}),                 # padded to 128
     _left(1, 1, 6, 5, 5, 0, 10.0, 1.0, softcap=1.0, mask={"size": 1, "keep_first": 3}),                       # no rotation, itself and three
     _left(2, 1, 128, 64, 3, 128, 300.0, 0.05),                                                                # no cap, no mask
@@ -270,19 +270,20 @@ def test_long_decoding_past_the_window_with_the_pages_dealt_to_several_workgroup
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("window,keep,dim,vdim", [(40, 20, 16, 12), (64, 64, 64, 64), (65, 3, 64, 128), (7, 70, 8, 12)])
+@pytest.mark.parametrize("window,keep,dim,vdim", [(36, 12, 16, 12), (64, 64, 64, 64), (65, 3, 64, 128), (7, 70, 8, 12)])
 def test_a_key_that_stands_out_at_every_edge_of_the_mask(lib, dtype, window, keep, dim, vdim):
     """The query's own input is also given to one earlier token, and keys are made from the matrix that makes queries, so that
-    this token's key takes the query's softmax wherever the mask lets it: just inside and just outside the window, and as the
+    this token's key shares the query's softmax with the query's own key wherever the mask lets it: just inside and just outside the window, and as the
     last kept token and the first that is not kept, in a prompt and in decoding.  One tap, no biases, strong norms."""
     hidden = 64
-    p = _left(2, 1, dim, vdim, 1, 2, 1000.0, 8.0 / dim, softcap=30.0, mask={"size": window, "keep_first": keep})
+    p = _left(2, 1, dim, vdim, 1, 2, 1000.0, 8.0 / dim, softcap=40.0, mask={"size": window, "keep_first": keep})
     w = _left_weights(hidden, p, seed=window)
     w["k"] = w["q"][:dim].clone()
     for name, rows in (("q", 2 * dim), ("k", dim), ("v", vdim)):
         w[name + ".b"] = torch.zeros(rows, dtype=F64)
         w[name + ".conv"] = torch.ones(rows, 1, dtype=F64)
-    w["q.norm"] = w["k.norm"] = torch.full((dim,), 1.5, dtype=F64)
+    w["q.norm"] = w["k.norm"] = torch.full((dim,), 2.0, dtype=F64)
+    w["q.norm"][:2] = 0.125                  # the rotated pair turns by a radian a token: it is kept small, so that the copy's score is the query's own
     part = _left_part(lib, hidden, p, dtype)
     part.load(_place(part, w, dtype))
     t_len = keep + window + 70
@@ -293,9 +294,9 @@ def test_a_key_that_stands_out_at_every_edge_of_the_mask(lib, dtype, window, kee
         q = P.norm_plain((x @ w["q"].T).view(t_len, 2, dim), w["q.norm"], EPS)
         k = P.norm_plain((x @ w["k"].T).view(t_len, 1, dim), w["k.norm"], EPS)
         f = P.frequencies(2, 1000.0)
-        a = P.attention_weights(P.rotate(q, f, "halves"), P.rotate(k, f, "halves"), p["scale"], P.visible(t_len, window, keep), 30.0)
+        a = P.attention_weights(P.rotate(q, f, "halves"), P.rotate(k, f, "halves"), p["scale"], P.visible(t_len, window, keep), 40.0)
         if seen:
-            assert float(a[0, query, at]) > 0.05                    # the edge shows in the plain weights
+            assert float(a[0, query, at]) > 0.3                     # the edge shows in the plain weights
         else:
             assert float(a[:, query, at].max()) == 0.0
         want = P.windowed_attention(x, w, p, EPS)
@@ -393,10 +394,10 @@ def _ff(ff, limit):
 
 # everything different from layer to layer; the parallel layer first; layers that run another layer's weights between others
 MODEL_A = {"architecture": "Menerax", "vocab": 96, "width": 64, "norm": {"eps": 1e-5}, "layers": [
-    {"type": "parallel", "mixer": _par(_left(4, 2, 16, 24, 3, 8, 100.0, 0.3, softcap=6.0, mask={"size": 40, "keep_first": 10}), 2, 16, 4, 0.6, 1.1),
+    {"type": "parallel", "mixer": _par(_left(4, 2, 16, 24, 3, 8, 100.0, 0.3, softcap=6.0, mask={"size": 44, "keep_first": 10}), 2, 16, 4, 0.55, 1.2),
      "mlp": _ff(96, 1.0)},
     {"type": "latent_attention", "mixer": _lat(3, 8, 4, 6, 12, 10, 0.3, 100.0), "mlp": None},
-    {"type": "parallel", "mixer": _par(_left(4, 2, 16, 24, 3, 8, 100.0, 0.3, softcap=6.0, mask={"size": 40, "keep_first": 10}), 2, 16, 4, 0.6, 1.1),
+    {"type": "parallel", "mixer": _par(_left(4, 2, 16, 24, 3, 8, 100.0, 0.3, softcap=6.0, mask={"size": 44, "keep_first": 10}), 2, 16, 4, 0.55, 1.2),
      "mlp": _ff(96, 1.0), "weights_of": 0},
     {"type": "latent_attention", "mixer": _lat(4, 16, 8, 12, 24, 40, 0.2, 5e4), "mlp": _ff(40, 0.5)},
     {"type": "parallel", "mixer": _par(_left(2, 1, 8, 8, 2, 8, 5e5, 0.4, mask={"size": 9, "keep_first": 0},
@@ -412,8 +413,8 @@ MODEL_B = {"architecture": "Menerax", "vocab": 50, "width": 32, "norm": {"eps": 
 # sizes on the matrix cores' grid: 128 numbers a token through the latent, heads of 64 and 128, a window of whole pages
 MODEL_C = {"architecture": "Menerax", "vocab": 320, "width": 128, "norm": {"eps": 1e-5}, "layers": [
     {"type": "latent_attention", "mixer": _lat(8, 32, 32, 32, 64, 96, 0.12, 1e4), "mlp": _ff(256, 2.0)},
-    {"type": "parallel", "mixer": _par(_left(8, 2, 64, 64, 4, 32, 5e5, 0.125, softcap=30.0, mask={"size": 128, "keep_first": 64},
-                                              scaling={"factor": 8.0, "low": 1.0, "high": 4.0, "original": 256}), 2, 64, 16, 0.5, 1.2),
+    {"type": "parallel", "mixer": _par(_left(8, 2, 64, 64, 4, 32, 2e5, 0.11, softcap=25.0, mask={"size": 128, "keep_first": 64},
+                                              scaling={"factor": 6.0, "low": 1.0, "high": 3.0, "original": 256}), 2, 64, 16, 0.5, 1.2),
      "mlp": _ff(128, 1.5)},
     {"type": "latent_attention", "mixer": _lat(8, 32, 32, 32, 64, 96, 0.12, 1e4), "mlp": _ff(256, 2.0), "weights_of": 0},
     {"type": "parallel", "mixer": _par(_left(4, 4, 128, 64, 3, 64, 1e4, 0.09, softcap=10.0, mask={"size": 70, "keep_first": 5}), 4, 32, 8, 1.0, 0.7),
@@ -572,17 +573,17 @@ def _random_config(rng):
     def parallel():
         dim, kvh, group = rng.choice([8, 16, 32, 64, 128]), rng.choice([1, 2, 4]), rng.choice([1, 2, 3, 4, 8, 20])
         dims = rng.choice([0, 2, dim // 2, dim])
-        rot = {"base": rng.choice([1e4, 5e5]), "dims": dims - dims % 2}
+        rot = {"base": rng.choice([1e4, 2e5]), "dims": dims - dims % 2}
         if rot["dims"] and rng.random() < 0.5:
-            rot["scaling"] = {"factor": rng.choice([2.0, 8.0]), "low": 1.0, "high": rng.choice([2.0, 4.0]), "original": rng.choice([16, 64, 2048])}
+            rot["scaling"] = {"factor": rng.choice([2.0, 6.0]), "low": 1.0, "high": rng.choice([2.0, 3.0]), "original": rng.choice([16, 64, 1024])}
         left = dict(heads=kvh * group, kv_heads=kvh, dim=dim, vdim=rng.choice([8, 16, 48, 64, 128]), conv=rng.choice([1, 2, 3, 4, 7]), rot=rot,
                     scale=rng.choice([0.1, 0.125, 0.3]))
         if rng.random() < 0.8:
-            left["softcap"] = rng.choice([5.0, 30.0, 50.0])
+            left["softcap"] = rng.choice([5.0, 25.0, 50.0])
         if rng.random() < 0.85:
-            left["mask"] = {"size": rng.choice([1, 7, 40, 64, 100, 128, 200]), "keep_first": rng.choice([0, 1, 4, 20, 64, 70, 130])}
+            left["mask"] = {"size": rng.choice([1, 7, 36, 64, 100, 128, 200]), "keep_first": rng.choice([0, 1, 4, 12, 64, 70, 130])}
         right = dict(heads=rng.choice([1, 2, 6, 8]), dim=rng.choice([8, 16, 32, 64]), decay_rank=rng.choice([1, 4, 16, 24]))
-        return {"left": left, "right": right, "left_scale": rng.choice([0.6, 1.0, 1.5]), "right_scale": rng.choice([0.4, 1.1])}
+        return {"left": left, "right": right, "left_scale": rng.choice([0.5, 1.0, 1.5]), "right_scale": rng.choice([0.4, 1.2])}
 
     layers = []
     for _ in range(rng.choice([2, 3, 4])):
